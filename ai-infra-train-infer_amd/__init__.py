@@ -1,0 +1,31 @@
+"""MI355X (gfx950) paged-attention hot path for the ai-infra-train-infer inference engine.
+
+Exports the names a caller would import from the reference's src/inference package for
+this path (src/inference/__init__.py:18-68): the context functions, the KV tensors of the
+block pool, store_kv_cache and the two attention modules.  Compute is done by hand-written
+HIP kernels behind a C ABI (include/paged_attn.h, libpaged_attn.so next to this file).
+
+The directory name contains a hyphen, so import it through the `ai_infra_train_infer_amd`
+loader module at the repository root.
+"""
+from .context import InferenceContext, set_context, get_context, reset_context
+from .kv_cache import BlockPool, HAS_FP8, _FP8_DTYPE
+from .attention import (
+    PagedAttention,
+    PartitionedPagedAttention,
+    store_kv_cache,
+    paged_decode,
+    paged_prefill,
+    choose_partition,
+    HAS_FLASH_ATTN,
+    HAS_TRITON,
+)
+from . import _native
+
+__all__ = [
+    "InferenceContext", "set_context", "get_context", "reset_context",
+    "BlockPool", "HAS_FP8",
+    "PagedAttention", "PartitionedPagedAttention", "store_kv_cache",
+    "paged_decode", "paged_prefill", "choose_partition",
+    "HAS_FLASH_ATTN", "HAS_TRITON",
+]

@@ -1,0 +1,332 @@
+"""Paged attention ops and modules backed by the gfx950 HIP kernels.
+
+Same names, argument order and defaults as the reference's src/inference/attention.py
+(store_kv_cache :44-72, PagedAttention :188-382, PartitionedPagedAttention :387-626), so a model
+runner that binds caches by isinstance() and sets the global context can use these classes
+unchanged.  Everything computes on the GPU through libpaged_attn.so; a CPU tensor or a
+missing library raises RuntimeError (there is no fallback path).
+"""
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import _native
+from .context import get_context
+from .kv_cache import HAS_FP8, _FP8_DTYPE
+
+# Probe flags kept for callers that import them from the reference module.  Neither
+# flash-attn nor Triton is used here.
+HAS_FLASH_ATTN = False
+HAS_TRITON = False
+
+_DTYPE_CODE = {
+    torch.float16: _native.DTYPE_F16,
+    torch.bfloat16: _native.DTYPE_BF16,
+    torch.float32: _native.DTYPE_F32,
+}
+if HAS_FP8:
+    _DTYPE_CODE[_FP8_DTYPE] = _native.DTYPE_FP8_E4M3
+
+
+def _code(dtype, what):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError("%s: unsupported dtype %s" % (what, dtype)) from None
+
+
+def _require_gpu(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(
+            "%s: tensor is on %s; the paged-attention kernels run on the GPU only and this "
+            "package has no CPU path" % (what, t.device))
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _rows(t, what):
+    """[N, H, D] tensor with contiguous (H, D) -> (tensor, token stride in elements)."""
+    if t.dim() != 3:
+        raise RuntimeError("%s: expected [tokens, heads, head_dim], got %s" % (what, tuple(t.shape)))
+    if t.stride(2) != 1 or t.stride(1) != t.shape[2] or (t.shape[0] > 1 and t.stride(0) < t.shape[1] * t.shape[2]):
+        t = t.contiguous()
+    return t, (t.stride(0) if t.shape[0] > 1 else t.shape[1] * t.shape[2])
+
+
+def _int32(t, what):
+    if t.dtype != torch.int32:
+        t = t.to(torch.int32)
+    if not t.is_contiguous():
+        t = t.contiguous()
+    return t
+
+
+def _check_cache(k_cache, v_cache, what):
+    if k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise RuntimeError("%s: caches must both be [num_blocks, block_size, kv_heads, head_dim]" % what)
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("%s: cache layer views must be contiguous" % what)
+    if k_cache.dtype != v_cache.dtype:
+        raise RuntimeError("%s: k_cache and v_cache dtypes differ" % what)
+
+
+# ==================== KV cache write ====================
+
+def store_kv_cache(
+    key: torch.Tensor,
+    value: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    k_scale: Optional[torch.Tensor] = None,
+    v_scale: Optional[torch.Tensor] = None,
+    cache_dtype: str = "fp16",
+):
+    """Write new K/V rows into their physical cache slots.
+
+    key, value   [num_tokens, num_kv_heads, head_dim]
+    k_cache/v_cache  [num_blocks, block_size, num_kv_heads, head_dim] (one layer)
+    slot_mapping [num_tokens] int32, slot = block_id * block_size + offset, negative = skip
+    k_scale/v_scale  [num_blocks, block_size] fp32, fp8 mode only
+    cache_dtype  "fp16" (bit copy in the cache dtype) or "fp8" (per-token 448/amax quantisation)
+
+    Dispatch follows src/inference/attention.py:67-72: fp8 when requested and available,
+    otherwise the copy.
+    """
+    _require_gpu(key, "store_kv_cache")
+    _require_gpu(k_cache, "store_kv_cache")
+    _check_cache(k_cache, v_cache, "store_kv_cache")
+    lib = _native.load()
+    num_blocks, block_size, num_kv_heads, head_dim = k_cache.shape
+    total_slots = num_blocks * block_size
+    row = num_kv_heads * head_dim
+    n = key.shape[0]
+    if value.shape != key.shape or tuple(key.shape[1:]) != (num_kv_heads, head_dim):
+        raise RuntimeError("store_kv_cache: key/value shape %s/%s does not match the cache %s"
+                           % (tuple(key.shape), tuple(value.shape), tuple(k_cache.shape)))
+    if slot_mapping.numel() != n:
+        raise RuntimeError("store_kv_cache: slot_mapping has %d entries for %d tokens"
+                           % (slot_mapping.numel(), n))
+    if n == 0:
+        return
+    key, ks = _rows(key, "store_kv_cache")
+    value, vs = _rows(value, "store_kv_cache")
+    slots = _int32(slot_mapping, "store_kv_cache")
+    stream = _stream_ptr(key.device)
+
+    if cache_dtype == "fp8" and HAS_FP8:
+        if k_cache.dtype != _FP8_DTYPE:
+            raise RuntimeError("store_kv_cache: cache_dtype='fp8' needs float8_e4m3fn caches, got %s"
+                               % k_cache.dtype)
+        if k_scale is None or v_scale is None:
+            raise RuntimeError("store_kv_cache: fp8 mode needs k_scale and v_scale")
+        if (k_scale.numel() != total_slots or v_scale.numel() != total_slots
+                or k_scale.dtype != torch.float32 or v_scale.dtype != torch.float32
+                or not k_scale.is_contiguous() or not v_scale.is_contiguous()):
+            raise RuntimeError("store_kv_cache: scales must be contiguous fp32 [num_blocks, block_size]")
+        if value.dtype != key.dtype:
+            raise RuntimeError("store_kv_cache: key and value dtypes differ")
+        rc = lib.pa_kv_store_fp8(key.data_ptr(), value.data_ptr(), _code(key.dtype, "store_kv_cache"),
+                                 ks, vs, k_cache.data_ptr(), v_cache.data_ptr(),
+                                 k_scale.data_ptr(), v_scale.data_ptr(), slots.data_ptr(), n, row,
+                                 total_slots, stream)
+        _native.check(rc, "pa_kv_store_fp8")
+    else:
+        if key.dtype != k_cache.dtype or value.dtype != v_cache.dtype:
+            # the reference's index_put_ refuses mixed dtypes as well
+            raise RuntimeError("store_kv_cache: key/value dtype %s does not match the cache dtype %s"
+                               % (key.dtype, k_cache.dtype))
+        rc = lib.pa_kv_store(key.data_ptr(), value.data_ptr(), ks, vs, k_cache.data_ptr(),
+                             v_cache.data_ptr(), slots.data_ptr(), n, row, key.element_size(),
+                             total_slots, stream)
+        _native.check(rc, "pa_kv_store")
+
+
+# ==================== decode launcher ====================
+
+_WORKSPACES = {}
+
+
+def _workspace(device, nbytes):
+    """Per (device, stream) scratch for the partition partials; grows, never shrinks."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+# workgroups the decode launch should reach before it stops splitting the context
+_TARGET_WORKGROUPS = 2048
+_MIN_AUTO_PARTITION = 256
+
+
+def choose_partition(batch, num_q_heads, num_kv_heads, max_context):
+    """Partition size for a decode launch that has no caller-given one.
+
+    batch * (query-head groups) workgroups alone fill the GPU at large batch; below that the
+    context is split into power-of-two partitions of at least 256 tokens until about
+    _TARGET_WORKGROUPS workgroups exist.  Returns (partition_size, max_partitions); (0, 1)
+    means a single pass.
+    """
+    g = num_q_heads // num_kv_heads
+    units = batch * (num_q_heads // (2 if g % 2 == 0 else 1))
+    if units >= _TARGET_WORKGROUPS or max_context <= _MIN_AUTO_PARTITION:
+        return 0, 1
+    p = _MIN_AUTO_PARTITION
+    while p * 2 < max_context and units * ((max_context + 2 * p - 1) // (2 * p)) >= _TARGET_WORKGROUPS:
+        p *= 2
+    parts = (max_context + p - 1) // p
+    if parts <= 1:
+        return 0, 1
+    return p, parts
+
+
+def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale=None,
+                 v_scale=None, partition_size=None, out=None):
+    """Decode attention of q [batch, heads, head_dim] against the paged cache.
+
+    partition_size None: single pass, or an automatic split when the batch alone cannot fill
+    the GPU (same result up to fp32 rounding).  partition_size > 0: the partitioned algorithm
+    of src/inference/attention.py:434-626 with that size.  Never synchronises with the host.
+    """
+    _require_gpu(q, "paged_decode")
+    _require_gpu(k_cache, "paged_decode")
+    _check_cache(k_cache, v_cache, "paged_decode")
+    lib = _native.load()
+    if q.dim() != 3:
+        raise RuntimeError("paged_decode: q must be [batch, heads, head_dim]")
+    batch, num_q_heads, head_dim = q.shape
+    num_blocks, block_size, num_kv_heads, d2 = k_cache.shape
+    if d2 != head_dim:
+        raise RuntimeError("paged_decode: q head_dim %d != cache head_dim %d" % (head_dim, d2))
+    if block_tables.dim() != 2 or block_tables.shape[0] != batch or context_lens.numel() != batch:
+        raise RuntimeError("paged_decode: block_tables/context_lens do not match the batch")
+    q, qs = _rows(q, "paged_decode")
+    tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+    if tables.stride(1) != 1:
+        tables = tables.contiguous()
+    lens = _int32(context_lens, "paged_decode")
+    if out is None:
+        out = torch.empty((batch, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+    if batch == 0:
+        return out
+    kv_code = _code(k_cache.dtype, "paged_decode")
+    fp8 = kv_code == _native.DTYPE_FP8_E4M3
+    if fp8 and (k_scale is None or v_scale is None):
+        raise RuntimeError("paged_decode: fp8 cache needs k_scale and v_scale")
+    max_context = tables.shape[1] * block_size
+    if partition_size is None:
+        psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context)
+    else:
+        psize = int(partition_size)
+        parts = max(1, (max_context + psize - 1) // psize)
+    ws_ptr, ws_bytes = None, 0
+    if parts > 1:
+        ws_bytes = lib.pa_workspace_bytes(batch, num_q_heads, head_dim, parts)
+        ws = _workspace(q.device, ws_bytes)
+        ws_ptr = ws.data_ptr()
+    rc = lib.pa_decode(q.data_ptr(), _code(q.dtype, "paged_decode"), qs, k_cache.data_ptr(),
+                       v_cache.data_ptr(), k_scale.data_ptr() if fp8 else None,
+                       v_scale.data_ptr() if fp8 else None, kv_code, tables.data_ptr(),
+                       tables.stride(0), lens.data_ptr(), out.data_ptr(), out.stride(0), batch,
+                       num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, float(scale),
+                       psize, parts, ws_ptr, ws_bytes, _stream_ptr(q.device))
+    _native.check(rc, "pa_decode")
+    return out
+
+
+def paged_prefill(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, scale,
+                  block_tables=None, k_scale=None, v_scale=None, out=None):
+    """Causal varlen prefill.  With block_tables, K/V come from the paged cache (cached prefix
+    + new chunk, bottom-right aligned mask); without, from the dense new-token tensors."""
+    raise NotImplementedError("paged_prefill: the MFMA prefill kernel is not built yet")
+
+
+# ==================== modules ====================
+
+class PagedAttention(nn.Module):
+    """Attention layer of the inference engine: writes the new K/V into the paged cache, then
+    runs varlen prefill or single-token decode according to the global context.
+
+    k_cache / v_cache / k_scale / v_scale / cache_dtype are bound by the model runner
+    (src/inference/model_runner.py:102-116).
+    """
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int,
+                 cache_dtype: str = "fp16"):
+        super().__init__()
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.scale = head_dim ** -0.5
+        self.cache_dtype = cache_dtype
+        self.k_cache: Optional[torch.Tensor] = None
+        self.v_cache: Optional[torch.Tensor] = None
+        self.k_scale: Optional[torch.Tensor] = None
+        self.v_scale: Optional[torch.Tensor] = None
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        """q [tokens, heads, dim], k/v [tokens, kv_heads, dim] -> [tokens, heads, dim]."""
+        ctx = get_context()
+        # the write precedes the read: context_lens already counts the new token
+        if self.k_cache is not None and ctx.slot_mapping is not None:
+            store_kv_cache(k, v, self.k_cache, self.v_cache, ctx.slot_mapping,
+                           k_scale=self.k_scale, v_scale=self.v_scale,
+                           cache_dtype=self.cache_dtype)
+        if ctx.is_prefill:
+            return self._prefill_attention(q, k, v, ctx)
+        return self._decode_attention(q, ctx)
+
+    def _scales(self):
+        if self.cache_dtype == "fp8" and self.k_scale is not None:
+            return self.k_scale, self.v_scale
+        return None, None
+
+    def _prefill_attention(self, q, k, v, ctx):
+        if ctx.block_tables is not None and self.k_cache is not None:
+            ks, vs = self._scales()
+            return paged_prefill(q, self.k_cache, self.v_cache, ctx.cu_seqlens_q, ctx.cu_seqlens_k,
+                                 ctx.max_seqlen_q, self.scale, block_tables=ctx.block_tables,
+                                 k_scale=ks, v_scale=vs)
+        return paged_prefill(q, k, v, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.max_seqlen_q,
+                             self.scale)
+
+    def _decode_attention(self, q, ctx):
+        if self.k_cache is None or ctx.block_tables is None or ctx.context_lens is None:
+            return q  # nothing bound: same last-resort behaviour as attention.py:329-330
+        ks, vs = self._scales()
+        return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
+                            self.scale, k_scale=ks, v_scale=vs)
+
+
+class PartitionedPagedAttention(PagedAttention):
+    """Decode attention split into partitions of `partition_size` tokens with an exact
+    log-sum-exp merge (src/inference/attention.py:387-626).
+
+    The reference picks the path after a host read of max(context_lens); here the launch is
+    sized from the block-table width instead, so no host synchronisation happens: sequences
+    shorter than one partition simply own a single partition, which merges to itself.
+    """
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int,
+                 cache_dtype: str = "fp16", partition_size: int = 512):
+        super().__init__(num_heads, num_kv_heads, head_dim, cache_dtype)
+        self.partition_size = partition_size
+
+    def _decode_attention(self, q, ctx):
+        if ctx.context_lens is None:
+            return super()._decode_attention(q, ctx)
+        return self._partitioned_decode(q, ctx)
+
+    def _partitioned_decode(self, q, ctx):
+        if self.k_cache is None or ctx.block_tables is None or ctx.context_lens is None:
+            return q
+        ks, vs = self._scales()
+        return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
+                            self.scale, k_scale=ks, v_scale=vs,
+                            partition_size=self.partition_size)

@@ -1,0 +1,86 @@
+"""Builds libpaged_attn.so (the C-ABI HIP library) for gfx950 with hipcc.
+
+Usage:  python build.py [--force]
+
+Each csrc/*.hip file is compiled to an object in csrc/_obj/ (in parallel) and the objects
+are linked into libpaged_attn.so next to this file.  hipcc cross-compiles for gfx950
+without a GPU present.  The library depends on the HIP runtime only (no torch symbols).
+"""
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+OBJ = os.path.join(CSRC, "_obj")
+LIB = os.path.join(HERE, "libpaged_attn.so")
+ARCH = "gfx950"
+
+# -packed-fp32-ops: keep hipcc from forming v_pk_{add,mul,fma}_f32 out of ordinary float code.
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
+            f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
+            "-I", INCLUDE, "-I", CSRC] + DEVICE_FLAGS
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or put /opt/rocm/bin on PATH)")
+
+
+def sources():
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _newest_input():
+    files = sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    files += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE)] + [os.path.abspath(__file__)]
+    return max(os.path.getmtime(f) for f in files)
+
+
+def is_current():
+    return os.path.exists(LIB) and os.path.getmtime(LIB) >= _newest_input()
+
+
+def _compile(hipcc, src):
+    obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+    cmd = [hipcc] + CXXFLAGS + ["-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-8000:]))
+    # the host pass does not know the device-only target feature; that warning is expected
+    noise = ("packed-fp32-ops", "is not a recognized feature")
+    msgs = [ln for ln in r.stderr.splitlines() if ln.strip() and not any(n in ln for n in noise)]
+    return obj, "\n".join(msgs)
+
+
+def build_library(force=True, verbose=False):
+    """Compile and link the library. With force=False an up-to-date library is kept."""
+    if not force and is_current():
+        return LIB
+    hipcc = _hipcc()
+    os.makedirs(OBJ, exist_ok=True)
+    srcs = sources()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        results = list(ex.map(lambda s: _compile(hipcc, s), srcs))
+    for obj, msgs in results:
+        if verbose and msgs:
+            print(msgs, file=sys.stderr)
+    objs = [o for o, _ in results]
+    tmp = LIB + ".tmp"
+    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", "-o", tmp] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+    os.replace(tmp, LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    path = build_library(force=True, verbose=True)
+    print(path)

@@ -1,0 +1,235 @@
+"""Benchmark of the paged decode attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload (BASELINE.json configs[1] shape, the one the metric is quoted on): batch 64, context
+4096 per sequence, 16 query / 8 KV heads, head_dim 128, block_size 16, block tables a random
+permutation of the pool, synthetic N(0,1) data.  One step = one paged decode attention call
+through the package's operator (the call PagedAttention._decode_attention makes once per
+layer), inputs resident in HBM.  The FP16-KV run gives `value` (achieved HBM GB/s on the
+algorithmic bytes); the FP8-KV run of the same shape is reported beside it.
+
+Prints ONE JSON line.  `roofline` is for the dominant kernel (the attention pass alone,
+timed with HIP events on the launch stream); `cpu_baseline` times the oracle (the
+reference's PyTorch fallback restated) on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def algorithmic_bytes(batch, ctx, hq, hkv, d, bs, fp8):
+    """K and V of every context token once, fp8 scales, q in and out, table entries and lens."""
+    e = 1 if fp8 else 2
+    kv = batch * ctx * hkv * d * 2 * e
+    scales = batch * ctx * 2 * 4 if fp8 else 0
+    qo = 2 * batch * hq * d * 2
+    meta = batch * ((ctx + bs - 1) // bs) * 4 + batch * 4
+    return kv + scales + qo + meta
+
+
+def build_workload(pa, torch, dev, batch, ctx, hq, hkv, d, bs, fp8, seed):
+    """Pool, tables and query generated on the GPU (seeded); fp8 pools are produced by the
+    quantising store kernel so the bytes read are the ones the writer makes."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    blocks_per_seq = (ctx + bs - 1) // bs
+    nb = batch * blocks_per_seq + 64
+    perm = torch.randperm(nb, generator=g, device=dev)[:batch * blocks_per_seq]
+    tables = perm.view(batch, blocks_per_seq).to(torch.int32).contiguous()
+    lens = torch.full((batch,), ctx, dtype=torch.int32, device=dev)
+    q = torch.randn(batch, hq, d, generator=g, device=dev, dtype=torch.float32).half()
+    if not fp8:
+        k_cache = torch.randn(nb, bs, hkv, d, generator=g, device=dev, dtype=torch.float32).half()
+        v_cache = torch.randn(nb, bs, hkv, d, generator=g, device=dev, dtype=torch.float32).half()
+        return dict(q=q, k_cache=k_cache, v_cache=v_cache, k_scale=None, v_scale=None,
+                    block_tables=tables, context_lens=lens, num_blocks=nb)
+    k_cache = torch.zeros(nb, bs, hkv, d, dtype=torch.float8_e4m3fn, device=dev)
+    v_cache = torch.zeros(nb, bs, hkv, d, dtype=torch.float8_e4m3fn, device=dev)
+    k_scale = torch.ones(nb, bs, dtype=torch.float32, device=dev)
+    v_scale = torch.ones(nb, bs, dtype=torch.float32, device=dev)
+    pos = torch.arange(ctx, device=dev)
+    for b in range(batch):
+        k = torch.randn(ctx, hkv, d, generator=g, device=dev, dtype=torch.float32).half()
+        v = torch.randn(ctx, hkv, d, generator=g, device=dev, dtype=torch.float32).half()
+        slots = (tables[b, pos // bs].long() * bs + pos % bs).to(torch.int32)
+        pa.store_kv_cache(k, v, k_cache, v_cache, slots, k_scale, v_scale, "fp8")
+    return dict(q=q, k_cache=k_cache, v_cache=v_cache, k_scale=k_scale, v_scale=v_scale,
+                block_tables=tables, context_lens=lens, num_blocks=nb)
+
+
+def time_steps(torch, fn, steps, warmup):
+    """W untimed + K timed calls on the current stream; returns (ms per step by HIP events,
+    ms per step by the host clock around synchronised ends)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return start.elapsed_time(stop) / steps, (t1 - t0) * 1e3 / steps
+
+
+def cpu_baseline(torch, w, scale, sample_seqs, bs, repeats=3):
+    """The oracle's decode (per-sequence gather + SDPA on the host) over the first
+    `sample_seqs` sequences of the workload, compacted into a small pool."""
+    from oracle import paged_attention_oracle as oracle
+    tables = w["block_tables"][:sample_seqs]
+    flat = tables.reshape(-1).long()
+    k = w["k_cache"][flat].cpu()
+    v = w["v_cache"][flat].cpu()
+    ks = w["k_scale"][flat].cpu() if w["k_scale"] is not None else None
+    vs = w["v_scale"][flat].cpu() if w["v_scale"] is not None else None
+    new_tables = torch.arange(flat.numel(), dtype=torch.int32).view(tables.shape)
+    q = w["q"][:sample_seqs].cpu()
+    lens = w["context_lens"][:sample_seqs].cpu()
+    kind = "fp8" if ks is not None else "fp16"
+    oracle.decode(q, k, v, new_tables, lens, scale, ks, vs, kind)        # warm-up
+    best = float("inf")
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        out = oracle.decode(q, k, v, new_tables, lens, scale, ks, vs, kind)
+        best = min(best, time.perf_counter() - t0)
+    return best, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--ctx", type=int, default=4096)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-seqs", type=int, default=8)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures the single-GPU hot path only; --gpus %d is not "
+              "supported (the path shards by sequence or KV head with no exchange)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ai_infra_train_infer_amd as pa
+    lib = pa._native.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, CTX, HQ, HKV, D, BS = args.batch, args.ctx, 16, 8, 128, 16
+    scale = 1.0 / math.sqrt(D)
+    results = {}
+    for kind in ("fp16", "fp8"):
+        fp8 = kind == "fp8"
+        w = build_workload(pa, torch, dev, B, CTX, HQ, HKV, D, BS, fp8, seed=1002)
+        out = torch.empty(B, HQ, D, dtype=torch.float16, device=dev)
+
+        def step():
+            pa.paged_decode(w["q"], w["k_cache"], w["v_cache"], w["block_tables"],
+                            w["context_lens"], scale, w["k_scale"], w["v_scale"], out=out)
+
+        ev_ms, wall_ms = time_steps(torch, step, args.steps, args.warmup)
+
+        # dominant kernel alone: the attention pass without the merge
+        psize, parts = pa.choose_partition(B, HQ, HKV, w["block_tables"].shape[1] * BS)
+        nbytes = lib.pa_workspace_bytes(B, HQ, D, parts)
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        kv_code = pa._native.DTYPE_FP8_E4M3 if fp8 else pa._native.DTYPE_F16
+        ksp = w["k_scale"].data_ptr() if fp8 else None
+        vsp = w["v_scale"].data_ptr() if fp8 else None
+
+        def kernel_only():
+            rc = lib.pa_decode_partials(w["q"].data_ptr(), 0, HQ * D, w["k_cache"].data_ptr(),
+                                        w["v_cache"].data_ptr(), ksp, vsp, kv_code,
+                                        w["block_tables"].data_ptr(), w["block_tables"].stride(0),
+                                        w["context_lens"].data_ptr(), B, HQ, HKV, D, BS,
+                                        w["num_blocks"], scale, max(psize, 16), parts, ws.data_ptr(),
+                                        ws.numel(), stream)
+            assert rc == 0, lib.pa_last_error()
+
+        k_ms, _ = time_steps(torch, kernel_only, args.steps, args.warmup)
+        nbytes_alg = algorithmic_bytes(B, CTX, HQ, HKV, D, BS, fp8)
+        results[kind] = dict(us_per_step=ev_ms * 1e3, wall_us_per_step=wall_ms * 1e3,
+                             kernel_us=k_ms * 1e3, bytes=nbytes_alg,
+                             gbps=nbytes_alg / (ev_ms * 1e-3) / 1e9,
+                             kernel_gbps=nbytes_alg / (k_ms * 1e-3) / 1e9,
+                             partition_size=psize, partitions=parts)
+        if kind == "fp16" and not args.no_cpu_baseline:
+            n = min(args.cpu_sample_seqs, B)
+            sec, cpu_out = cpu_baseline(torch, w, scale, n, BS)
+            step()
+            torch.cuda.synchronize()
+            err = float((out[:n].cpu().float() - cpu_out.float()).abs().max())
+            sample_bytes = algorithmic_bytes(n, CTX, HQ, HKV, D, BS, False)
+            results["cpu"] = dict(value=sample_bytes / sec / 1e9, unit="GB/s",
+                                  cores=torch.get_num_threads(), kind="port",
+                                  sample="oracle decode (per-sequence gather + SDPA) of the first %d of %d "
+                                         "sequences, ctx %d, FP16 KV, best of 3: %.1f ms; "
+                                         "host has %d logical CPUs; max |gpu-cpu| on the sample %.2e"
+                                         % (n, B, CTX, sec * 1e3, os.cpu_count(), err),
+                                  us_per_step_extrapolated=sec * 1e6 * B / n)
+        del w
+        torch.cuda.empty_cache()
+
+    f16, f8 = results["fp16"], results["fp8"]
+    line = {
+        "metric": "paged decode attn achieved HBM GB/s (% peak) + us/step at bs=64 ctx=4k",
+        "value": round(f16["gbps"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(f16["us_per_step"] / 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 accumulate over f16 KV (fp8-e4m3 KV reported beside it)",
+        "data": "synthetic N(0,1), seeded, random-permutation block tables",
+        "config": {
+            "workload": "BASELINE configs[1] shape: paged decode attention, batch %d, ctx %d, 16 q / 8 kv "
+                        "heads, head_dim 128, block_size 16, FP16 KV for `value`" % (B, CTX),
+            "partition_size": f16["partition_size"], "partitions": f16["partitions"],
+            "waves_per_workgroup": lib.pa_get_decode_waves(),
+        },
+        "pct_hbm_peak": round(100.0 * f16["gbps"] / HBM_PEAK_GBPS, 2),
+        "us_per_step": round(f16["us_per_step"], 2),
+        "wall_us_per_step": round(f16["wall_us_per_step"], 2),
+        "fp8": {
+            "us_per_step": round(f8["us_per_step"], 2),
+            "gbps": round(f8["gbps"], 1),
+            "pct_hbm_peak": round(100.0 * f8["gbps"] / HBM_PEAK_GBPS, 2),
+            "kernel_us": round(f8["kernel_us"], 2),
+            "speedup_vs_fp16": round(f16["us_per_step"] / f8["us_per_step"], 3),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "paged_decode_kernel<f16, 128, 2, W> (attention pass without the merge)",
+            "achieved": round(f16["kernel_gbps"], 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(f16["kernel_gbps"] / HBM_PEAK_GBPS, 4),
+            "kernel_us": round(f16["kernel_us"], 2),
+            "algorithmic_bytes": f16["bytes"],
+            "traffic": None,
+        },
+    }
+    if "cpu" in results:
+        line["cpu_baseline"] = results["cpu"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

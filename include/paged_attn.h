@@ -1,0 +1,208 @@
+/*
+ * paged_attn.h — C ABI of the MI355X (gfx950) paged-attention library.
+ *
+ * Every entry point takes raw device pointers, plain integer sizes and a HIP
+ * stream handle (void*, a hipStream_t; NULL = the default stream).  Nothing
+ * here allocates or frees device memory, synchronises with the host, or keeps
+ * a pointer after returning: the caller owns every buffer.  All launches are
+ * asynchronous on `stream` and may be recorded into a HIP graph.
+ *
+ * Return value: PA_OK (0) or a negative PA_ERR_* code; pa_last_error() then
+ * holds a message for the calling thread.
+ *
+ * Data layout (the reference engine's, kept as is):
+ *   K or V cache of one layer  [num_blocks, block_size, num_kv_heads, head_dim]
+ *                              contiguous, fp16 / bf16 / fp8-e4m3fn
+ *                              (reference: src/inference/kv_cache.py:131-174,
+ *                               bound per layer at src/inference/model_runner.py:102-116)
+ *   k_scale / v_scale          [num_blocks, block_size] fp32, one multiplier per token
+ *                              (448 / amax; dequant = fp8 / scale)
+ *   slot_mapping               [num_tokens] int32, slot = block_id*block_size + offset,
+ *                              negative = skip (src/inference/attention.py:94,132,155)
+ *   block_tables               [batch, bt_stride] int32, entries past
+ *                              ceil(context_len/block_size) are never dereferenced
+ *   context_lens               [batch] int32, 0 = padded row (output row is zeroed)
+ */
+#ifndef PAGED_ATTN_H_
+#define PAGED_ATTN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_OK 0
+#define PA_ERR_BAD_ARG (-1)      /* null pointer, negative size, misaligned buffer */
+#define PA_ERR_UNSUPPORTED (-2)  /* shape or dtype the kernels are not built for */
+#define PA_ERR_LAUNCH (-3)       /* hipGetLastError() reported a failure */
+#define PA_ERR_WORKSPACE (-4)    /* workspace missing or too small */
+
+/* element types */
+#define PA_DTYPE_F16 0
+#define PA_DTYPE_BF16 1
+#define PA_DTYPE_F32 2
+#define PA_DTYPE_FP8_E4M3 3 /* OCP e4m3fn, the layout of torch.float8_e4m3fn */
+
+/* Library ABI version (bumped when a signature changes). */
+int pa_version(void);
+
+/* Message for the last non-zero return code on this thread ("" if none). */
+const char* pa_last_error(void);
+
+/*
+ * Paged KV-cache write, same-dtype bit copy.
+ * Replaces: store_kv_cache -> _store_kv_cache_pytorch / _store_kv_cache_triton
+ *           (src/inference/attention.py:44-72, 119-135, 141-183).
+ * For every token t with 0 <= slot_mapping[t] < total_slots the row
+ * key[t, :row_elems] is copied to k_cache[slot, :row_elems] (same for value).
+ * Negative slots are skipped; slots >= total_slots are skipped too (the
+ * reference would raise an index error on the host).
+ *   key/value            [num_tokens, row_elems], token stride given in elements
+ *   row_elems            num_kv_heads * head_dim; row_elems*elem_bytes % 16 == 0
+ *   elem_bytes           1, 2 or 4
+ */
+int pa_kv_store(const void* key, const void* value, int64_t key_token_stride,
+                int64_t value_token_stride, void* k_cache, void* v_cache,
+                const int32_t* slot_mapping, int64_t num_tokens, int64_t row_elems,
+                int elem_bytes, int64_t total_slots, void* stream);
+
+/*
+ * Paged KV-cache write with per-token FP8-e4m3fn quantisation.
+ * Replaces: store_kv_cache -> _store_kv_cache_fp8 (src/inference/attention.py:75-116).
+ * Per token and per tensor: amax = max |fp32(x)| over the row, clamped to >= 1e-5;
+ * s = fl(fl(1/amax) * 448) in fp32 (how torch evaluates the reference's `448.0 / amax`:
+ * reciprocal, then multiply, each correctly rounded); byte = e4m3fn(fp32(x) * s) with
+ * round-to-nearest-even and no saturation; bytes go to the cache row, s to
+ * the scale slot.  Bytes and scales are bit-identical to the reference arithmetic.
+ *   in_dtype             PA_DTYPE_F16 / BF16 / F32
+ *   row_elems            num_kv_heads * head_dim, a multiple of 16
+ */
+int pa_kv_store_fp8(const void* key, const void* value, int in_dtype,
+                    int64_t key_token_stride, int64_t value_token_stride, void* k_cache,
+                    void* v_cache, float* k_scale, float* v_scale,
+                    const int32_t* slot_mapping, int64_t num_tokens, int64_t row_elems,
+                    int64_t total_slots, void* stream);
+
+/*
+ * Bytes of workspace for `max_partitions` partitions (per-partition max, sum and
+ * normalised partial output, all fp32).  pa_decode with max_partitions == 1 needs no
+ * workspace at all; pa_decode_partials / pa_merge always do.
+ */
+int64_t pa_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t head_dim,
+                           int64_t max_partitions);
+
+/*
+ * Paged decode attention: one query token per sequence against its paged context.
+ * Replaces: PagedAttention._decode_attention / _sdpa_decode_fallback
+ *           (src/inference/attention.py:263-279, 317-382) when max_partitions == 1, and
+ *           PartitionedPagedAttention._partitioned_decode_fallback with
+ *           _compute_partition_attention + _merge_partitions
+ *           (src/inference/attention.py:434-626) when max_partitions > 1.
+ *
+ * out[b, h, :] = softmax_j(scale * q[b,h,:] . K[b,j,h/G,:]) @ V[b,:,h/G,:] over the
+ * first context_lens[b] tokens found through block_tables[b].  fp8 caches are
+ * dequantised as fp8 / scale[slot].  Accumulation is fp32.
+ *
+ * max_partitions == 1: single pass, result written straight to `out`.
+ * max_partitions  > 1: partition p of sequence b covers tokens
+ *   [p*partition_size, min((p+1)*partition_size, context_len)); the last partition
+ *   (p == max_partitions-1) absorbs whatever lies beyond it, so a context longer than
+ *   max_partitions*partition_size is still computed exactly.  Per partition the
+ *   kernel stores max (natural-log units), sum of exp and the locally normalised
+ *   output into `workspace`; the merge reduction then writes `out`.
+ *
+ *   q, out               [batch, num_q_heads, head_dim], token stride in elements
+ *   q_dtype              PA_DTYPE_F16 / BF16 / F32 (out has the same type)
+ *   kv_dtype             PA_DTYPE_F16 / BF16 / FP8_E4M3
+ *   k_scale, v_scale     required for fp8, ignored otherwise
+ *   num_blocks           blocks in the pool (block ids are clamped to it)
+ *   head_dim             64 or 128;  block_size a power of two >= 8
+ *   partition_size       a multiple of 16 (ignored when max_partitions == 1)
+ *   workspace            >= pa_workspace_bytes(...) bytes, 256-byte aligned
+ */
+int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+              const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
+              const int32_t* block_tables, int64_t bt_stride, const int32_t* context_lens,
+              void* out, int64_t out_token_stride, int64_t batch, int64_t num_q_heads,
+              int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+              float scale, int64_t partition_size, int64_t max_partitions, void* workspace,
+              int64_t workspace_bytes, void* stream);
+
+/*
+ * First half of the partitioned decode only: fills `workspace` and does not merge.
+ * Replaces: the loop over _compute_partition_attention
+ *           (src/inference/attention.py:462-470, 519-589).
+ * Workspace layout (fp32):  max [batch, num_q_heads, max_partitions]
+ *                           sum [batch, num_q_heads, max_partitions]
+ *                           out [batch, num_q_heads, max_partitions, head_dim]
+ * Partition lse = max + log(sum).  Entries of partitions past the context are not written.
+ */
+int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+                       const void* v_cache, const float* k_scale, const float* v_scale,
+                       int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
+                       const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
+                       int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                       int64_t num_blocks, float scale, int64_t partition_size,
+                       int64_t max_partitions, void* workspace, int64_t workspace_bytes,
+                       void* stream);
+
+/*
+ * Merge reduction over partitions.
+ * Replaces: PartitionedPagedAttention._merge_partitions (src/inference/attention.py:591-626).
+ * out = sum_p w_p * out_p / sum_p w_p with w_p = sum_p * exp(max_p - max_all), over the
+ * min(ceil(context_len/partition_size), max_partitions) partitions of each sequence.
+ */
+int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* context_lens,
+             void* out, int out_dtype, int64_t out_token_stride, int64_t batch,
+             int64_t num_q_heads, int64_t head_dim, int64_t partition_size,
+             int64_t max_partitions, void* stream);
+
+/*
+ * Chunked-prefill paged attention (MFMA): every new token of a sequence attends to the
+ * cached prefix plus the new tokens up to itself, all read from the paged cache.
+ * Replaces: PagedAttention._prefill_attention with block_tables set, i.e.
+ *           flash_attn_varlen_func(..., causal=True, block_table=...)
+ *           (src/inference/attention.py:240-261); with no prefix it equals
+ *           _sdpa_prefill_fallback (src/inference/attention.py:281-315).
+ * Row i of sequence s (i in [0, Lq_s)) sees keys [0, Lk_s - Lq_s + i] (bottom-right
+ * aligned causal mask), Lq_s = cu_seqlens_q[s+1]-cu_seqlens_q[s],
+ * Lk_s = cu_seqlens_k[s+1]-cu_seqlens_k[s] (cached + new tokens).
+ *   q, out               [total_q_tokens, num_q_heads, head_dim]
+ *   cu_seqlens_q/k       [num_seqs + 1] int32 (InferenceContext.cu_seqlens_q / cu_seqlens_k)
+ *   block_tables         [num_seqs, bt_stride]; NULL = K/V are dense [total_k_tokens,
+ *                        num_kv_heads, head_dim] tensors indexed by cu_seqlens_k (no prefix
+ *                        hit: the reference then passes the new k, v themselves)
+ *   max_seqlen_q         upper bound of Lq_s (sizes the launch grid)
+ */
+int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+               const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
+               const int32_t* block_tables, int64_t bt_stride, const int32_t* cu_seqlens_q,
+               const int32_t* cu_seqlens_k, void* out, int64_t out_token_stride,
+               int64_t num_seqs, int64_t max_seqlen_q, int64_t num_q_heads,
+               int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+               float scale, void* stream);
+
+/*
+ * fp8-e4m3fn -> fp32 conversion of n bytes (the in-register dequant step of the
+ * attention kernels, exposed for checking the cache contents).
+ * Replaces: `ki.to(torch.float16)` before the divide (src/inference/attention.py:361-362).
+ */
+int pa_fp8_e4m3_to_f32(const void* src, float* dst, int64_t n, void* stream);
+
+/*
+ * fp32 -> fp8-e4m3fn conversion of n values with the cache writer's rounding
+ * (round-to-nearest-even, no saturation, NaN = 0x7F).
+ * Replaces: `.to(torch.float8_e4m3fn)` (src/inference/attention.py:109-110).
+ */
+int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
+
+/* Tunables of the decode launch (waves per workgroup: 1, 2, 4 or 8). Returns PA_OK or BAD_ARG. */
+int pa_set_decode_waves(int waves_per_workgroup);
+int pa_get_decode_waves(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PAGED_ATTN_H_ */

@@ -1,0 +1,229 @@
+"""Paged decode attention on the GPU against the oracle (the reference's PyTorch paged
+attention restated on the CPU).  Tolerances are BASELINE's: rtol 1e-3 / atol 2e-3 for 16-bit
+caches, rtol 1e-2 / atol 1e-2 for fp8 caches."""
+import pytest
+import torch
+
+import cases
+from oracle import paged_attention_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+# bf16 has no stated tolerance: its 8-bit mantissa (output and oracle arithmetic) sets 2e-2 / 1e-2
+TOL = {"fp16": dict(rtol=1e-3, atol=2e-3), "bf16": dict(rtol=2e-2, atol=1e-2),
+       "fp8": dict(rtol=1e-2, atol=1e-2)}
+
+
+def oracle_decode(c):
+    return oracle.decode(c["q"], c["k_cache"], c["v_cache"], c["block_tables"], c["context_lens"],
+                         c["scale"], c["k_scale"], c["v_scale"], c["cache_dtype"])
+
+
+def gpu_decode(pa, c, gpu, partition_size=None):
+    d = cases.to_device(c, gpu)
+    out = pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                          d["scale"], d["k_scale"], d["v_scale"], partition_size=partition_size)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def check(got, want, kind):
+    assert not torch.isnan(got).any(), "NaN in the output: a read outside the context"
+    torch.testing.assert_close(got.float(), want.float(), **TOL[kind])
+
+
+def test_config1_fp16(pa, gpu):
+    c = cases.config1()
+    check(gpu_decode(pa, c, gpu), oracle_decode(c), "fp16")
+
+
+@pytest.mark.parametrize("waves", [1, 2, 4, 8])
+@pytest.mark.parametrize("cache", ["fp16", "fp8", "bf16"])
+def test_every_workgroup_width(pa, lib, gpu, waves, cache):
+    c = cases.make_case(40 + waves, [1, 15, 16, 17, 100, 333, 512, 47], 128, cache=cache,
+                        q_dtype=torch.bfloat16 if cache == "bf16" else torch.float16)
+    want = oracle_decode(c)
+    assert lib.pa_set_decode_waves(waves) == 0
+    try:
+        got_single = gpu_decode(pa, c, gpu)
+        got_part = gpu_decode(pa, c, gpu, partition_size=64)
+    finally:
+        lib.pa_set_decode_waves(4)
+    check(got_single, want, cache)
+    check(got_part, want, cache)
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(16, 8, 128), (8, 8, 128), (32, 8, 128), (16, 2, 64),
+                                       (4, 4, 64), (12, 4, 128)])
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_head_shapes(pa, gpu, hq, hkv, d, cache):
+    c = cases.make_case(hq * 3 + d, [5, 64, 129, 700], 96, num_heads=hq, num_kv_heads=hkv,
+                        head_dim=d, cache=cache)
+    check(gpu_decode(pa, c, gpu), oracle_decode(c), cache)
+
+
+@pytest.mark.parametrize("bs", [8, 32, 128])
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_block_sizes(pa, gpu, bs, cache):
+    lens = [1, bs - 1, bs, bs + 1, 5 * bs + 3, 301]
+    c = cases.make_case(bs, lens, 64, block_size=bs, cache=cache)
+    want = oracle_decode(c)
+    check(gpu_decode(pa, c, gpu), want, cache)
+    check(gpu_decode(pa, c, gpu, partition_size=48), want, cache)
+
+
+@pytest.mark.parametrize("qdt", [torch.float32, torch.bfloat16])
+def test_query_dtypes_against_fp64(pa, gpu, qdt):
+    c = cases.make_case(77, [33, 260, 17], 40, q_dtype=qdt)
+    got = gpu_decode(pa, c, gpu)
+    assert got.dtype == qdt
+    want = oracle.decode_f64(c["q"], c["k_cache"], c["v_cache"], c["block_tables"],
+                             c["context_lens"], c["scale"])
+    torch.testing.assert_close(got.double(), want, rtol=1e-3 if qdt == torch.float32 else 1e-2,
+                               atol=2e-3 if qdt == torch.float32 else 1e-2)
+    check(got, oracle_decode(c), "fp16" if qdt == torch.float32 else "fp8")
+
+
+def test_fp32_query_is_accurate_to_fp32_level(pa, gpu):
+    c = cases.make_case(78, [200, 31], 32, q_dtype=torch.float32)
+    got = gpu_decode(pa, c, gpu).double()
+    want = oracle.decode_f64(c["q"], c["k_cache"], c["v_cache"], c["block_tables"],
+                             c["context_lens"], c["scale"])
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("pad", [-1, 0, 123456])
+def test_padding_rows_and_garbage_table_tails(pa, gpu, pad):
+    c = cases.make_case(11, [0, 40, 0, 16, 250], 64, pad=pad, extra_cols=5)
+    got = gpu_decode(pa, c, gpu)
+    assert float(got[0].abs().max()) == 0.0 and float(got[2].abs().max()) == 0.0
+    check(got, oracle_decode(c), "fp16")
+    gotp = gpu_decode(pa, c, gpu, partition_size=32)
+    assert float(gotp[0].abs().max()) == 0.0
+    check(gotp, oracle_decode(c), "fp16")
+
+
+def test_ctx1_returns_the_single_value_row(pa, gpu):
+    c = cases.make_case(12, [1, 1, 1, 1], 8)
+    got = gpu_decode(pa, c, gpu)
+    for b in range(4):
+        blk = int(c["block_tables"][b, 0])
+        for h in range(16):
+            assert torch.equal(got[b, h], c["v_cache"][blk, 0, h // 2])
+
+
+def test_strided_query_and_preallocated_output(pa, gpu):
+    c = cases.make_case(13, [90, 300], 40)
+    d = cases.to_device(c, gpu)
+    wide = torch.zeros(2, 16 * 128 + 256, dtype=torch.float16, device=gpu)
+    wide[:, :16 * 128] = d["q"].view(2, -1)
+    qv = wide[:, :16 * 128].view(2, 16, 128)
+    out = torch.empty(2, 16, 128, dtype=torch.float16, device=gpu)
+    res = pa.paged_decode(qv, d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                          d["scale"], out=out)
+    torch.cuda.synchronize()
+    assert res is out
+    check(out.cpu(), oracle_decode(c), "fp16")
+
+
+def test_config2_fp8_headline_shape(pa, gpu):
+    c = cases.config2()
+    got = gpu_decode(pa, c, gpu)
+    check(got, oracle_decode(c), "fp8")
+    # the same launch through the explicit 512-token partitioning
+    check(gpu_decode(pa, c, gpu, partition_size=512), oracle_decode(c), "fp8")
+
+
+def test_config2_fp8_per_tensor_scale(pa, gpu):
+    c = cases.config2(seed=2002, batch=8, ctx=4096, per_tensor_scale=True)
+    check(gpu_decode(pa, c, gpu), oracle_decode(c), "fp8")
+
+
+def test_config2_shape_fp16(pa, gpu):
+    c = cases.config2(seed=1102, cache="fp16", batch=16)
+    check(gpu_decode(pa, c, gpu), oracle_decode(c), "fp16")
+
+
+def test_config3_partitioned_long_context(pa, gpu):
+    c = cases.config3()
+    want = oracle_decode(c)                      # single-pass reference, as the config asks
+    check(gpu_decode(pa, c, gpu, partition_size=512), want, "fp16")
+    check(gpu_decode(pa, c, gpu), want, "fp16")   # automatic split
+
+
+def test_config4_shared_prefix(pa, gpu):
+    c = cases.config4()
+    t = c["block_tables"]
+    assert torch.equal(t[1, :64], t[0, :64]) and torch.equal(t[15, :64], t[8, :64])
+    check(gpu_decode(pa, c, gpu), oracle_decode(c), "fp16")
+
+
+def test_partials_match_the_reference_partition_outputs(pa, lib, gpu):
+    c = cases.make_case(31, [700, 64, 1030], 160, q_dtype=torch.float32)
+    d = cases.to_device(c, gpu)
+    B, H, D, P = 3, 16, 128, 256
+    parts = (d["block_tables"].shape[1] * 16 + P - 1) // P
+    nbytes = lib.pa_workspace_bytes(B, H, D, parts)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=gpu)
+    rc = lib.pa_decode_partials(d["q"].data_ptr(), 2, H * D, d["k_cache"].data_ptr(),
+                                d["v_cache"].data_ptr(), None, None, 0, d["block_tables"].data_ptr(),
+                                d["block_tables"].stride(0), d["context_lens"].data_ptr(), B, H, 8, D,
+                                16, c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, None)
+    assert rc == 0, lib.pa_last_error()
+    out = torch.empty(B, H, D, dtype=torch.float32, device=gpu)
+    rc = lib.pa_merge(ws.data_ptr(), nbytes, d["context_lens"].data_ptr(), out.data_ptr(), 2, H * D,
+                      B, H, D, P, parts, None)
+    assert rc == 0, lib.pa_last_error()
+    torch.cuda.synchronize()
+    rows = B * H * parts
+    scal = ((rows * 4 + 255) // 256) * 256
+    wsc = ws.cpu()
+    mx = wsc[:rows * 4].view(torch.float32).view(B, H, parts)
+    sm = wsc[scal:scal + rows * 4].view(torch.float32).view(B, H, parts)
+    po = wsc[2 * scal:2 * scal + rows * D * 4].view(torch.float32).view(B, H, parts, D)
+    for b in range(B):
+        n = int(c["context_lens"][b])
+        for p in range((n + P - 1) // P):
+            o, lse = oracle.partition_attention(c["q"][b:b + 1], c["k_cache"], c["v_cache"],
+                                                c["block_tables"][b], p * P, min((p + 1) * P, n), 16,
+                                                c["scale"])
+            torch.testing.assert_close(po[b, :, p], o[0], rtol=1e-4, atol=1e-5)
+            torch.testing.assert_close(mx[b, :, p] + torch.log(sm[b, :, p]), lse[0], rtol=1e-5, atol=1e-5)
+    check(out.cpu(), oracle_decode(c), "fp16")
+
+
+def test_more_partitions_than_workspace_rows_still_exact(pa, lib, gpu):
+    # max_partitions smaller than ceil(ctx/P): the last partition absorbs the rest
+    c = cases.make_case(32, [900, 100], 80)
+    d = cases.to_device(c, gpu)
+    B, H, D, P, parts = 2, 16, 128, 128, 3
+    nbytes = lib.pa_workspace_bytes(B, H, D, parts)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=gpu)
+    out = torch.empty(B, H, D, dtype=torch.float16, device=gpu)
+    rc = lib.pa_decode(d["q"].data_ptr(), 0, H * D, d["k_cache"].data_ptr(), d["v_cache"].data_ptr(),
+                       None, None, 0, d["block_tables"].data_ptr(), d["block_tables"].stride(0),
+                       d["context_lens"].data_ptr(), out.data_ptr(), H * D, B, H, 8, D, 16,
+                       c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, None)
+    assert rc == 0, lib.pa_last_error()
+    torch.cuda.synchronize()
+    check(out.cpu(), oracle_decode(c), "fp16")
+
+
+def test_c_abi_argument_errors(lib, gpu):
+    t = torch.zeros(16, dtype=torch.float16, device=gpu)
+    p = t.data_ptr()
+    base = dict(q=p, kc=p, vc=p, bt=p, cl=p, out=p)
+    def call(**kw):
+        a = dict(hq=16, hkv=8, d=128, bs=16, psize=0, parts=1, ws=None, wsb=0, kvd=0)
+        a.update(kw)
+        return lib.pa_decode(base["q"], 0, a["hq"] * a["d"], base["kc"], base["vc"], None, None,
+                             a["kvd"], base["bt"], 1, base["cl"], base["out"], a["hq"] * a["d"], 1,
+                             a["hq"], a["hkv"], a["d"], a["bs"], 4, 1.0, a["psize"], a["parts"],
+                             a["ws"], a["wsb"], None)
+    assert call(d=96) == -2 and b"head_dim" in lib.pa_last_error()
+    assert call(bs=12) == -2
+    assert call(bs=4) == -2
+    assert call(hq=15) == -1
+    assert call(kvd=3) == -1                      # fp8 without scales
+    assert call(parts=4, psize=500, ws=p, wsb=1 << 30) == -2      # not a multiple of 16
+    assert call(parts=4, psize=512) == -4         # workspace missing

@@ -1,0 +1,72 @@
+"""Host-side behaviour that needs no GPU: the context surface, launch-shape policy, and the
+refusal to compute anywhere but on the GPU."""
+import pytest
+import torch
+
+
+def test_context_set_get_reset(pa):
+    pa.reset_context()
+    c = pa.get_context()
+    assert c.is_prefill is False and c.slot_mapping is None and c.block_tables is None
+    sm = torch.zeros(3, dtype=torch.int32)
+    pa.set_context(False, slot_mapping=sm, context_lens=sm, block_tables=sm.view(3, 1))
+    c2 = pa.get_context()
+    assert c2 is not c and c2.slot_mapping is sm and c2.max_seqlen_q == 0
+    pa.set_context(True, cu_seqlens_q=sm, cu_seqlens_k=sm, max_seqlen_q=5, max_seqlen_k=9)
+    assert pa.get_context().is_prefill and pa.get_context().max_seqlen_k == 9
+    assert pa.get_context().slot_mapping is None        # replaced, not mutated
+    pa.reset_context()
+    assert pa.get_context().cu_seqlens_q is None
+
+
+def test_module_surface_matches_reference_names(pa):
+    m = pa.PagedAttention(16, 8, 128)
+    assert (m.num_heads, m.num_kv_heads, m.head_dim, m.cache_dtype) == (16, 8, 128, "fp16")
+    assert m.scale == 128 ** -0.5 and m.k_cache is None and m.k_scale is None
+    p = pa.PartitionedPagedAttention(16, 8, 128, "fp8")
+    assert p.partition_size == 512 and p.cache_dtype == "fp8" and isinstance(p, pa.PagedAttention)
+    assert pa.HAS_FLASH_ATTN is False and pa.HAS_TRITON is False and pa.HAS_FP8 is True
+
+
+def test_decode_without_bound_cache_returns_q(pa):
+    pa.set_context(False, context_lens=torch.ones(2, dtype=torch.int32))
+    q = torch.randn(2, 16, 128)
+    assert pa.PagedAttention(16, 8, 128)(q, q[:, :8], q[:, :8]) is q
+    assert pa.PartitionedPagedAttention(16, 8, 128)(q, q[:, :8], q[:, :8]) is q
+    pa.reset_context()
+
+
+def test_cpu_tensors_are_refused_not_emulated(pa):
+    k = torch.zeros(2, 8, 128, dtype=torch.float16)
+    cache = torch.zeros(4, 16, 8, 128, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pa.store_kv_cache(k, k, cache, cache.clone(), torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pa.paged_decode(torch.zeros(2, 16, 128, dtype=torch.float16), cache, cache,
+                        torch.zeros(2, 1, dtype=torch.int32), torch.ones(2, dtype=torch.int32), 1.0)
+
+
+def test_choose_partition_policy(pa):
+    # batch fills the GPU on its own -> single pass
+    assert pa.choose_partition(512, 16, 8, 4096) == (0, 1)
+    # headline shape: 512 head groups, split until ~2048 workgroups
+    p, n = pa.choose_partition(64, 16, 8, 4096)
+    assert p % 16 == 0 and n == (4096 + p - 1) // p and 64 * 8 * n >= 2048
+    # long context, tiny batch: many partitions, each at least 256 tokens
+    p, n = pa.choose_partition(4, 16, 8, 32768)
+    assert p >= 256 and n * p >= 32768
+    # short context never splits
+    assert pa.choose_partition(1, 16, 8, 256) == (0, 1)
+
+
+def test_block_pool_layout(pa):
+    pool = pa.BlockPool(4, 16, 2, 8, 128, dtype=torch.float16, device="cpu", cache_dtype="fp8")
+    assert tuple(pool.kv_cache_tensor.shape) == (2, 2, 4, 16, 8, 128)
+    assert pool.kv_cache_tensor.dtype == torch.float8_e4m3fn
+    assert tuple(pool.k_scale.shape) == (2, 4, 16) and float(pool.k_scale.min()) == 1.0
+    assert tuple(pool.get_flattened_kv_cache().shape) == (2, 2, 64, 8, 128)
+    k, v, ks, vs = pool.layer_views(1)
+    assert k.is_contiguous() and v.data_ptr() - k.data_ptr() == 2 * 4 * 16 * 8 * 128
+    model = torch.nn.Sequential(pa.PagedAttention(16, 8, 128), pa.PartitionedPagedAttention(16, 8, 128))
+    assert pool.bind_to_model(model) == 2
+    assert model[1].k_cache.data_ptr() == k.data_ptr() and model[1].cache_dtype == "fp8"
