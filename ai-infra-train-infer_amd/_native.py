@@ -47,6 +47,7 @@ SIGNATURES = {
     "pa_f32_to_fp8_e4m3": (_int, [_ptr, _ptr, _i64, _ptr]),
     "pa_set_decode_waves": (_int, [_int]),
     "pa_get_decode_waves": (_int, []),
+    "pa_set_decode_pair_heads": (_int, [_int]),
 }
 
 _lock = threading.Lock()

@@ -160,21 +160,27 @@ def _workspace(device, nbytes):
     return ws
 
 
-# workgroups the decode launch should reach before it stops splitting the context
-_TARGET_WORKGROUPS = 2048
+# Workgroups the decode launch should reach before it stops splitting the context: one
+# 4-wave workgroup per CU (256 CUs) already keeps 8 KiB per wave in flight on every SIMD, and a
+# launch of that size runs as a single round with no merge pass (measured: splitting the
+# batch-64 / ctx-4096 launch further only adds the merge and the partial traffic).
+_TARGET_WORKGROUPS = 256
 _MIN_AUTO_PARTITION = 256
 
 
-def choose_partition(batch, num_q_heads, num_kv_heads, max_context):
+def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2):
     """Partition size for a decode launch that has no caller-given one.
 
-    batch * (query-head groups) workgroups alone fill the GPU at large batch; below that the
-    context is split into power-of-two partitions of at least 256 tokens until about
-    _TARGET_WORKGROUPS workgroups exist.  Returns (partition_size, max_partitions); (0, 1)
-    means a single pass.
+    One workgroup serves the query heads of one KV head (two heads of a GQA group at a time),
+    or of two adjacent KV heads when a head's row is 128 bytes or less.  If batch x those head
+    groups already give _TARGET_WORKGROUPS workgroups the launch is a single pass; otherwise the
+    context is split into power-of-two partitions of at least 256 tokens until about that many
+    exist.  Returns (partition_size, max_partitions); (0, 1) means a single pass.
     """
     g = num_q_heads // num_kv_heads
-    units = batch * (num_q_heads // (2 if g % 2 == 0 else 1))
+    gc = 2 if g % 2 == 0 else 1
+    hpw = 2 if (head_dim * kv_elem_bytes <= 128 and g == gc and num_kv_heads % 2 == 0) else 1
+    units = batch * (num_q_heads // (gc * hpw))
     if units >= _TARGET_WORKGROUPS or max_context <= _MIN_AUTO_PARTITION:
         return 0, 1
     p = _MIN_AUTO_PARTITION
@@ -221,7 +227,8 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale
         raise RuntimeError("paged_decode: fp8 cache needs k_scale and v_scale")
     max_context = tables.shape[1] * block_size
     if partition_size is None:
-        psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context)
+        psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim,
+                                        k_cache.element_size())
     else:
         psize = int(partition_size)
         parts = max(1, (max_context + psize - 1) // psize)

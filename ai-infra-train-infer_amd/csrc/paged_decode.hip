@@ -15,9 +15,9 @@
 //    fp16 row; the second half is the lane's second load).  No byte is fetched twice, so
 //    there is nothing for LDS to reuse in the main loop; LDS only carries the final
 //    cross-wave reduction.
-//  * Wave w of W walks tiles w, w+W, ... of 16 tokens (two row loads).  The loads of the next
-//    tile and the table entries of the one after are issued before the current tile is
-//    consumed, which keeps 8 KiB (fp16) per wave in flight.
+//  * Wave w of W walks tiles w, w+W, ... of 16 tokens (fp16/bf16: two row loads) or 32 tokens
+//    (fp8: four row loads).  The loads of the next tile and the table entries of the one after
+//    are issued before the current tile is consumed, which keeps 8 KiB per wave in flight.
 //  * q.K partial dots are reduced over the 8 lanes of a row with three DPP adds; each row
 //    group keeps its own running max / sum / output slice (no cross-lane traffic in the
 //    loop) and the groups are merged once at the end through LDS.
@@ -59,7 +59,7 @@ struct DecodeParams {
   float scale_log2e;
 };
 
-template <int KV, int D>
+template <int KV, int D, int HPW = 1>
 struct Geo {
   static constexpr int ES = (KV == KV_FP8) ? 1 : 2;  // bytes per cache element
   static constexpr int LPR = 8;                       // lanes per token row
@@ -69,6 +69,11 @@ struct Geo {
   static constexpr int NLD = BPL / LB;                // loads per lane per token
   static constexpr int WPT = BPL / 4;                 // dwords per lane per token
   static constexpr int EPC = LB / ES;                 // elements per load
+  // row loads (8 tokens each) per register tile: sized so a tile is 32 dwords of K + 32 of V
+  // per lane at most, i.e. 16 tokens of fp16 or 32 tokens of fp8 at head_dim 128
+  static constexpr int RL = (16 / WPT) < 4 ? (16 / WPT) : 4;
+  static constexpr int RPL = 8 / HPW;                 // token rows per row load
+  static constexpr int TILE = RPL * RL;               // tokens per tile
   static_assert(LB == 16 || LB == 8, "unsupported row geometry");
   // head-dim index of the lane's k-th element: loads are interleaved so that the 8 lanes of
   // a row cover LPR*LB contiguous bytes per load instruction.
@@ -111,40 +116,54 @@ __device__ __forceinline__ void unpack(const uint32_t (&w)[WPT], float (&x)[EPL]
   }
 }
 
-template <int KV, int D>
+template <int KV, int D, int HPW>
 struct Tile {
-  using G = Geo<KV, D>;
-  uint32_t k[2][G::WPT];
-  uint32_t v[2][G::WPT];
-  float ks[2];
-  float vs[2];
+  using G = Geo<KV, D, HPW>;
+  uint32_t k[G::RL][G::WPT];
+  uint32_t v[G::RL][G::WPT];
+  float ks[G::RL];
+  float vs[G::RL];
 };
 
-template <int KV, int D, int GC, int W>
+// HPW = KV heads per wavefront.  With HPW == 2 the 8-lane row groups alternate between two
+// adjacent KV heads, so 16 consecutive lanes read 2 x (head_dim * element size) contiguous
+// bytes: rows of 128 bytes or less (fp8 at head_dim 128, anything at head_dim 64) are then
+// fetched as 256-byte pieces, which HBM serves about 10% faster than lone 128-byte lines.
+template <int KV, int D, int GC, int W, int HPW>
 __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams p) {
-  using G = Geo<KV, D>;
+  using G = Geo<KV, D, HPW>;
+  using TileT = Tile<KV, D, HPW>;
   constexpr int EPL = G::EPL;
-  constexpr int NG = W * 4;  // partial outputs that reach LDS (row groups, pairwise pre-summed)
+  constexpr int RL = G::RL;
+  constexpr int RPL = G::RPL;
+  constexpr int TILE = G::TILE;
+  constexpr int GCW = GC * HPW;  // query heads per workgroup
+  constexpr int NG = W * 4;      // partial outputs per head that reach LDS
   constexpr float NEG_INF = -INFINITY;
 
-  __shared__ float red[NG][GC * D];
-  __shared__ float sm[GC][W];
-  __shared__ float sl[GC][W];
+  __shared__ float red[NG][GCW * D];
+  __shared__ float sm[GCW][W];
+  __shared__ float sl[GCW][W];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int g = lane >> 3;
-  const int j = lane & 7;
+  const int g = lane >> 3;        // row group 0..7
+  const int j = lane & 7;         // position inside the row
+  const int hs = g % HPW;         // which of the wave's KV heads this row group reads
+  const int tr = g / HPW;         // token row inside a row load
+  // blockIdx.x (fastest) walks the head groups, so the workgroups that share a token row are
+  // dispatched together and land on different XCDs: each L2 fetches only its own head's bytes.
   const int b = blockIdx.z;
   const int part = blockIdx.y;
-  const int h0 = blockIdx.x * GC;
-  const int kvh = h0 / (p.num_q_heads / p.num_kv_heads);
+  const int h0 = blockIdx.x * GCW;                                   // first query head of the workgroup
+  const int kvh = h0 / (p.num_q_heads / p.num_kv_heads) + hs;       // this lane's KV head
+  const int hq = h0 + hs * GC;                                       // this lane's first query head
 
   const int ctx = p.context_lens[b];
   if (ctx <= 0) {
     // padded batch row: the output row is zero; the merge kernel does the same when partitioned
     if (p.direct_out && part == 0) {
-      for (int o = threadIdx.x; o < GC * D; o += W * 64)
+      for (int o = threadIdx.x; o < GCW * D; o += W * 64)
         store_from_f32(p.out, b * p.out_stride + (int64_t)h0 * D + o, p.q_dtype, 0.0f);
     }
     return;
@@ -160,7 +179,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   float qf[GC][EPL];
 #pragma unroll
   for (int h = 0; h < GC; ++h) {
-    const int64_t base = b * p.q_stride + (int64_t)(h0 + h) * D;
+    const int64_t base = b * p.q_stride + (int64_t)(hq + h) * D;
 #pragma unroll
     for (int k = 0; k < EPL; k += 8) {
       float x[8];
@@ -182,27 +201,28 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   const int bs_mask = (1 << p.bs_log2) - 1;
   const uint32_t token_bytes = (uint32_t)(p.num_kv_heads * D * G::ES);
   const uint32_t block_bytes = token_bytes << p.bs_log2;
-  const uint32_t lane_off = (uint32_t)((g * p.num_kv_heads + kvh) * D * G::ES + j * G::LB);
+  const uint32_t lane_off = (uint32_t)((tr * p.num_kv_heads + kvh) * D * G::ES + j * G::LB);
   const int32_t* bt_row = p.block_tables + b * p.bt_stride;
-  const int last_blk = (end - 1) >> p.bs_log2;
-  const int nfull = (end - begin) >> 4;          // whole 16-token tiles of the partition
-  const bool has_tail = ((end - begin) & 15) != 0;
+  // never index past the table row, even if a context length is larger than the row holds
+  const int last_blk = min((end - 1) >> p.bs_log2, max((int)p.bt_stride - 1, 0));
+  const int nfull = (end - begin) / TILE;        // whole tiles of the partition
+  const bool has_tail = ((end - begin) % TILE) != 0;
 
   // physical block ids of the two row loads of a tile (wave-uniform scalar loads)
-  auto load_ids = [&](int tile, int (&ids)[2]) {
+  auto load_ids = [&](int tile, int (&ids)[RL]) {
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int tok = begin + tile * 16 + r * 8;
+    for (int r = 0; r < RL; ++r) {
+      const int tok = begin + tile * TILE + r * RPL;
       const int blk = min(tok >> p.bs_log2, last_blk);
       ids[r] = bt_row[blk];
     }
   };
   // start the K/V (and scale) loads of a tile; ids are clamped to the pool so that a corrupt
   // table can never fault
-  auto issue = [&](Tile<KV, D>& t, int tile, const int (&ids)[2]) {
+  auto issue = [&](TileT& t, int tile, const int (&ids)[RL]) {
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int tok = begin + tile * 16 + r * 8;
+    for (int r = 0; r < RL; ++r) {
+      const int tok = begin + tile * TILE + r * RPL;
       const uint32_t phys = (uint32_t)min(max(ids[r], 0), p.num_blocks - 1);
       const uint32_t off = (uint32_t)(tok & bs_mask);
       const uint64_t base = (uint64_t)phys * block_bytes + off * token_bytes;
@@ -215,19 +235,21 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
       }
       if constexpr (KV == KV_FP8) {
         const uint64_t slot = ((uint64_t)phys << p.bs_log2) + off;
-        t.ks[r] = p.k_scale[slot + g];
-        t.vs[r] = p.v_scale[slot + g];
+        t.ks[r] = p.k_scale[slot + tr];
+        t.vs[r] = p.v_scale[slot + tr];
       }
     }
   };
 
-  auto consume = [&](Tile<KV, D>& t, int tile, auto masked_tag) {
+  auto consume = [&](TileT& t, int tile, auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    float s[2][GC];
-    bool valid[2] = {true, true};
+    float s[RL][GC];
+    bool valid[RL];
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      if constexpr (MASKED) valid[r] = (begin + tile * 16 + r * 8 + g) < end;
+    for (int r = 0; r < RL; ++r) valid[r] = true;
+#pragma unroll
+    for (int r = 0; r < RL; ++r) {
+      if constexpr (MASKED) valid[r] = (begin + tile * TILE + r * RPL + tr) < end;
       float kf[EPL];
       unpack<KV, G::WPT, EPL>(t.k[r], kf);
       float inv_ks = 1.0f;
@@ -250,7 +272,10 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
     bool changed = false;
 #pragma unroll
     for (int h = 0; h < GC; ++h) {
-      m_new[h] = fmaxf(m[h], fmaxf(s[0][h], s[1][h]));
+      float mt = s[0][h];
+#pragma unroll
+      for (int r = 1; r < RL; ++r) mt = fmaxf(mt, s[r][h]);
+      m_new[h] = fmaxf(m[h], mt);
       changed |= m_new[h] > m[h];
     }
     if (__builtin_amdgcn_ballot_w64(changed) != 0) {
@@ -265,7 +290,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
       }
     }
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
+    for (int r = 0; r < RL; ++r) {
       if constexpr (MASKED) {
         if (!valid[r]) {
 #pragma unroll
@@ -298,8 +323,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   const int n_mine = nfull > wave ? (nfull - wave + W - 1) / W : 0;
   auto tile_of = [&](int i) { return wave + i * W; };
   if (n_mine > 0) {
-    Tile<KV, D> ta, tb;
-    int ids_a[2], ids_b[2];
+    TileT ta, tb;
+    int ids_a[RL], ids_b[RL];
     load_ids(tile_of(0), ids_a);
     issue(ta, tile_of(0), ids_a);
     if (n_mine > 1) load_ids(tile_of(1), ids_b);
@@ -319,69 +344,76 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   }
   // ---- the partial last tile, masked, by the wave whose turn it is --------------------------------
   if (has_tail && (nfull % W) == wave) {
-    Tile<KV, D> tt;
-    int ids_t[2];
+    TileT tt;
+    int ids_t[RL];
     load_ids(nfull, ids_t);
     issue(tt, nfull, ids_t);
     consume(tt, nfull, std::true_type{});
   }
 
-  // ---- merge the W*8 row groups: common max, then plain sums (DPP, shuffles, LDS) ------------
-  // all 8 lanes of a row group hold the same m and l, so lanes 8 apart are the partners
+  // ---- merge the row groups: common max, then plain sums (DPP, shuffles, LDS) ----------------
+  // All 8 lanes of a row group hold the same m and l.  Groups of the same KV head differ in
+  // lane bits 3..5 (HPW == 1) or 4..5 (HPW == 2, where bit 3 selects the head).
+  const bool writer = (j == 0) && (tr == 0);  // lane 0, plus lane 8 when it owns the second head
 #pragma unroll
   for (int h = 0; h < GC; ++h) {
-    float wm = fmaxf(m[h], dpp_f32<0x128>(m[h]));  // row_ror:8 = lane ^ 8 inside a 16-lane row
+    float wm = m[h];
+    if constexpr (HPW == 1) wm = fmaxf(wm, dpp_f32<0x128>(wm));  // row_ror:8 = lane ^ 8
     wm = fmaxf(wm, __shfl_xor(wm, 16));
     wm = fmaxf(wm, __shfl_xor(wm, 32));
-    if (lane == 0) sm[h][wave] = wm;
+    if (writer) sm[hs * GC + h][wave] = wm;
   }
   __syncthreads();
   float mx[GC];
 #pragma unroll
   for (int h = 0; h < GC; ++h) {
-    float v = sm[h][0];
+    float v = sm[hs * GC + h][0];
 #pragma unroll
-    for (int i = 1; i < W; ++i) v = fmaxf(v, sm[h][i]);
+    for (int i = 1; i < W; ++i) v = fmaxf(v, sm[hs * GC + h][i]);
     mx[h] = v;  // finite: the partition holds at least one token
   }
 #pragma unroll
   for (int h = 0; h < GC; ++h) {
     const float w = __builtin_amdgcn_exp2f(m[h] - mx[h]);  // exp2(-inf) = 0 for idle groups
     float lw = l[h] * w;
-    lw += dpp_f32<0x128>(lw);
+    if constexpr (HPW == 1) lw += dpp_f32<0x128>(lw);
     lw += __shfl_xor(lw, 16);
     lw += __shfl_xor(lw, 32);
-    if (lane == 0) sl[h][wave] = lw;
+    if (writer) sl[hs * GC + h][wave] = lw;
 #pragma unroll
     for (int k = 0; k < EPL; k += 4) {
       float o4[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float a = acc[h][k + e] * w;
-        o4[e] = a + dpp_f32<0x128>(a);
+        float a = acc[h][k + e] * w;
+        if constexpr (HPW == 1) a += dpp_f32<0x128>(a);  // pre-sum the two groups of a 16-lane row
+        o4[e] = a;
       }
-      if ((g & 1) == 0)
-        *(float4*)&red[wave * 4 + (g >> 1)][h * D + G::dim_of(k, j)] =
+      if (HPW == 2 || (g & 1) == 0)
+        *(float4*)&red[wave * 4 + (g >> 1)][(hs * GC + h) * D + G::dim_of(k, j)] =
             make_float4(o4[0], o4[1], o4[2], o4[3]);
     }
   }
   __syncthreads();
-  for (int o = threadIdx.x; o < GC * D; o += W * 64) {
-    const int h = o / D;
-    const int d = o - h * D;
+  for (int o = threadIdx.x; o < GCW * D; o += W * 64) {
+    const int hh = o / D;  // query head relative to h0
+    const int d = o - hh * D;
     float num = 0.0f, den = 0.0f;
 #pragma unroll
     for (int i = 0; i < NG; ++i) num += red[i][o];
 #pragma unroll
-    for (int i = 0; i < W; ++i) den += sl[h][i];
+    for (int i = 0; i < W; ++i) den += sl[hh][i];
     const float res = num / den;
     if (p.direct_out) {
-      store_from_f32(p.out, b * p.out_stride + (int64_t)(h0 + h) * D + d, p.q_dtype, res);
+      store_from_f32(p.out, b * p.out_stride + (int64_t)(h0 + hh) * D + d, p.q_dtype, res);
     } else {
-      const int64_t row = ((int64_t)b * p.num_q_heads + h0 + h) * p.max_partitions + part;
+      const int64_t row = ((int64_t)b * p.num_q_heads + h0 + hh) * p.max_partitions + part;
       p.ws_out[row * D + d] = res;
       if (d == 0) {
-        p.ws_max[row] = mx[h] * 0.6931471805599453f;  // back to natural-log units
+        float mo = sm[hh][0];
+#pragma unroll
+        for (int i = 1; i < W; ++i) mo = fmaxf(mo, sm[hh][i]);
+        p.ws_max[row] = mo * 0.6931471805599453f;  // back to natural-log units
         p.ws_sum[row] = den;
       }
     }
@@ -419,6 +451,7 @@ __global__ void merge_partitions_kernel(const float* __restrict__ ws_max,
 }
 
 static int g_decode_waves = 4;
+static int g_decode_pair_heads = 1;
 
 struct Workspace {
   float* mx;
@@ -444,23 +477,38 @@ static Workspace ws_split(void* ws, int64_t batch, int64_t hq, int64_t maxp) {
   return w;
 }
 
-template <int KV, int D, int GC>
+template <int KV, int D, int GC, int HPW>
 static void launch_decode_w(const DecodeParams& p, dim3 grid, int waves, hipStream_t st) {
   switch (waves) {
-    case 1: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 1>), grid, dim3(64), 0, st, p); break;
-    case 2: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 2>), grid, dim3(128), 0, st, p); break;
-    case 8: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 8>), grid, dim3(512), 0, st, p); break;
-    default: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 4>), grid, dim3(256), 0, st, p); break;
+    case 1: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 1, HPW>), grid, dim3(64), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 2, HPW>), grid, dim3(128), 0, st, p); break;
+    case 8: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 8, HPW>), grid, dim3(512), 0, st, p); break;
+    default: hipLaunchKernelGGL((paged_decode_kernel<KV, D, GC, 4, HPW>), grid, dim3(256), 0, st, p); break;
   }
 }
 
+// true when a KV row of one head is at most 128 bytes, where pairing heads in a wave pays
+template <int KV, int D>
+constexpr bool narrow_rows() { return D * Geo<KV, D>::ES <= 128; }
+
+template <int KV, int D, int GC>
+static void launch_decode_h(const DecodeParams& p, dim3 grid, int waves, int hpw, hipStream_t st) {
+  if constexpr (narrow_rows<KV, D>()) {
+    if (hpw == 2) {
+      launch_decode_w<KV, D, GC, 2>(p, grid, waves, st);
+      return;
+    }
+  }
+  launch_decode_w<KV, D, GC, 1>(p, grid, waves, st);
+}
+
 template <int KV>
-static int launch_decode_kv(const DecodeParams& p, dim3 grid, int d, int gc, int waves,
+static int launch_decode_kv(const DecodeParams& p, dim3 grid, int d, int gc, int waves, int hpw,
                             hipStream_t st) {
-  if (d == 128 && gc == 2) launch_decode_w<KV, 128, 2>(p, grid, waves, st);
-  else if (d == 128 && gc == 1) launch_decode_w<KV, 128, 1>(p, grid, waves, st);
-  else if (d == 64 && gc == 2) launch_decode_w<KV, 64, 2>(p, grid, waves, st);
-  else if (d == 64 && gc == 1) launch_decode_w<KV, 64, 1>(p, grid, waves, st);
+  if (d == 128 && gc == 2) launch_decode_h<KV, 128, 2>(p, grid, waves, hpw, st);
+  else if (d == 128 && gc == 1) launch_decode_h<KV, 128, 1>(p, grid, waves, hpw, st);
+  else if (d == 64 && gc == 2) launch_decode_h<KV, 64, 2>(p, grid, waves, hpw, st);
+  else if (d == 64 && gc == 1) launch_decode_h<KV, 64, 1>(p, grid, waves, hpw, st);
   else return fail(PA_ERR_UNSUPPORTED, "pa_decode: head_dim must be 64 or 128");
   return PA_OK;
 }
@@ -564,12 +612,16 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   }
 
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)(num_q_heads / gc), (unsigned)max_partitions, (unsigned)batch);
+  // two adjacent KV heads per wave when one head's row is 128 bytes or less (and each KV head's
+  // query group is handled whole, so adjacent workgroup heads are adjacent KV heads)
+  const int es = kv == KV_FP8 ? 1 : 2;
+  const int hpw = (g_decode_pair_heads && head_dim * es <= 128 && g == gc && num_kv_heads % 2 == 0) ? 2 : 1;
+  dim3 grid((unsigned)(num_q_heads / (gc * hpw)), (unsigned)max_partitions, (unsigned)batch);
   int rc;
   switch (kv) {
-    case KV_F16: rc = launch_decode_kv<KV_F16>(p, grid, (int)head_dim, gc, g_decode_waves, st); break;
-    case KV_BF16: rc = launch_decode_kv<KV_BF16>(p, grid, (int)head_dim, gc, g_decode_waves, st); break;
-    default: rc = launch_decode_kv<KV_FP8>(p, grid, (int)head_dim, gc, g_decode_waves, st); break;
+    case KV_F16: rc = launch_decode_kv<KV_F16>(p, grid, (int)head_dim, gc, g_decode_waves, hpw, st); break;
+    case KV_BF16: rc = launch_decode_kv<KV_BF16>(p, grid, (int)head_dim, gc, g_decode_waves, hpw, st); break;
+    default: rc = launch_decode_kv<KV_FP8>(p, grid, (int)head_dim, gc, g_decode_waves, hpw, st); break;
   }
   if (rc != PA_OK) return rc;
   rc = check_launch(who);
@@ -650,3 +702,8 @@ extern "C" int pa_set_decode_waves(int waves) {
 }
 
 extern "C" int pa_get_decode_waves(void) { return g_decode_waves; }
+
+extern "C" int pa_set_decode_pair_heads(int enable) {
+  g_decode_pair_heads = enable ? 1 : 0;
+  return PA_OK;
+}

@@ -143,7 +143,8 @@ def main():
         ev_ms, wall_ms = time_steps(torch, step, args.steps, args.warmup)
 
         # dominant kernel alone: the attention pass without the merge
-        psize, parts = pa.choose_partition(B, HQ, HKV, w["block_tables"].shape[1] * BS)
+        psize, parts = pa.choose_partition(B, HQ, HKV, w["block_tables"].shape[1] * BS, D,
+                                           w["k_cache"].element_size())
         nbytes = lib.pa_workspace_bytes(B, HQ, D, parts)
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream

@@ -200,6 +200,9 @@ int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
 /* Tunables of the decode launch (waves per workgroup: 1, 2, 4 or 8). Returns PA_OK or BAD_ARG. */
 int pa_set_decode_waves(int waves_per_workgroup);
 int pa_get_decode_waves(void);
+/* Tunable: let one wavefront serve two adjacent KV heads when a head's row is <= 128 bytes
+ * (fp8 at head_dim 128, any dtype at head_dim 64).  On by default. */
+int pa_set_decode_pair_heads(int enable);
 
 #ifdef __cplusplus
 }

@@ -47,11 +47,11 @@ def test_cpu_tensors_are_refused_not_emulated(pa):
 
 
 def test_choose_partition_policy(pa):
-    # batch fills the GPU on its own -> single pass
-    assert pa.choose_partition(512, 16, 8, 4096) == (0, 1)
-    # headline shape: 512 head groups, split until ~2048 workgroups
-    p, n = pa.choose_partition(64, 16, 8, 4096)
-    assert p % 16 == 0 and n == (4096 + p - 1) // p and 64 * 8 * n >= 2048
+    # headline shape: 64 x 8 head groups = 512 workgroups fill the GPU on their own -> single pass
+    assert pa.choose_partition(64, 16, 8, 4096) == (0, 1)
+    # a quarter of that batch is split four ways
+    p, n = pa.choose_partition(16, 16, 8, 4096)
+    assert p % 16 == 0 and n == (4096 + p - 1) // p and 16 * 8 * n >= 256
     # long context, tiny batch: many partitions, each at least 256 tokens
     p, n = pa.choose_partition(4, 16, 8, 32768)
     assert p >= 256 and n * p >= 32768
