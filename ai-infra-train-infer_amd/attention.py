@@ -249,9 +249,64 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale
 
 def paged_prefill(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, scale,
                   block_tables=None, k_scale=None, v_scale=None, out=None):
-    """Causal varlen prefill.  With block_tables, K/V come from the paged cache (cached prefix
-    + new chunk, bottom-right aligned mask); without, from the dense new-token tensors."""
-    raise NotImplementedError("paged_prefill: the MFMA prefill kernel is not built yet")
+    """Causal varlen prefill attention on the MFMA kernel.
+
+    q [total_new_tokens, heads, head_dim]; cu_seqlens_q / cu_seqlens_k int32 [num_seqs + 1]
+    (new tokens, and cached + new tokens, per sequence).  With block_tables, k_src / v_src are
+    the paged caches [num_blocks, block_size, kv_heads, head_dim] and row i of a chunk sees the
+    cached prefix plus the chunk up to itself; without, they are the dense new-token tensors
+    [total_k_tokens, kv_heads, head_dim] (src/inference/attention.py:243-257).
+    """
+    _require_gpu(q, "paged_prefill")
+    _require_gpu(k_src, "paged_prefill")
+    lib = _native.load()
+    if q.dim() != 3:
+        raise RuntimeError("paged_prefill: q must be [tokens, heads, head_dim]")
+    total_q, num_q_heads, head_dim = q.shape
+    q, qs = _rows(q, "paged_prefill")
+    if out is None:
+        out = torch.empty((total_q, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+    if total_q == 0:
+        return out
+    cu_q = _int32(cu_seqlens_q, "paged_prefill")
+    cu_k = _int32(cu_seqlens_k, "paged_prefill")
+    num_seqs = cu_q.numel() - 1
+    if cu_k.numel() != num_seqs + 1:
+        raise RuntimeError("paged_prefill: cu_seqlens_q and cu_seqlens_k differ in length")
+    kv_code = _code(k_src.dtype, "paged_prefill")
+    fp8 = kv_code == _native.DTYPE_FP8_E4M3
+    if block_tables is not None:
+        _check_cache(k_src, v_src, "paged_prefill")
+        num_blocks, block_size, num_kv_heads, d2 = k_src.shape
+        tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+        if tables.stride(1) != 1:
+            tables = tables.contiguous()
+        bt_ptr, bt_stride = tables.data_ptr(), tables.stride(0)
+        if fp8 and (k_scale is None or v_scale is None):
+            raise RuntimeError("paged_prefill: fp8 cache needs k_scale and v_scale")
+        kp, vp = k_src, v_src
+    else:
+        if k_src.dim() != 3 or v_src.shape != k_src.shape or k_src.dtype != v_src.dtype:
+            raise RuntimeError("paged_prefill: dense k/v must both be [tokens, kv_heads, head_dim]")
+        kp, kstride = _rows(k_src, "paged_prefill")
+        vp, vstride = _rows(v_src, "paged_prefill")
+        if vstride != kstride:
+            vp = vp.contiguous()
+            kp = kp.contiguous()
+            kstride = kp.shape[1] * kp.shape[2]
+        num_kv_heads, d2 = kp.shape[1], kp.shape[2]
+        num_blocks, block_size = 1, 1
+        bt_ptr, bt_stride = None, kstride
+    if d2 != head_dim:
+        raise RuntimeError("paged_prefill: q head_dim %d != k/v head_dim %d" % (head_dim, d2))
+    rc = lib.pa_prefill(q.data_ptr(), _code(q.dtype, "paged_prefill"), qs, kp.data_ptr(),
+                        vp.data_ptr(), k_scale.data_ptr() if fp8 else None,
+                        v_scale.data_ptr() if fp8 else None, kv_code, bt_ptr, bt_stride,
+                        cu_q.data_ptr(), cu_k.data_ptr(), out.data_ptr(), out.stride(0), num_seqs,
+                        int(max_seqlen_q), num_q_heads, num_kv_heads, head_dim, block_size,
+                        num_blocks, float(scale), _stream_ptr(q.device))
+    _native.check(rc, "pa_prefill")
+    return out
 
 
 # ==================== modules ====================

@@ -1,6 +1,392 @@
-// Chunked-prefill paged attention (MFMA) — entry point.
+// Chunked-prefill paged attention for gfx950 on the MFMA matrix cores.
+//
+// Reference semantics: PagedAttention._prefill_attention (src/inference/attention.py:240-261):
+// flash_attn_varlen_func(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, causal=True,
+// block_table=...) where K/V come from the paged cache when a prefix is cached, else from the
+// new tokens themselves; the causal mask is bottom-right aligned (row i of a chunk of Lq rows
+// sees keys 0 .. Lk-Lq+i).  Without a prefix this is _sdpa_prefill_fallback (:281-315).
+//
+// Here QK^T and PV are real dense tiles, so they run on v_mfma_f32_32x32x16_f16 with fp32
+// accumulation:
+//
+//  * One workgroup (4 waves) owns 128 query rows that share one KV head: 64 tokens x the two
+//    query heads of a GQA pair (or 128 tokens x 1 head).  Each wave owns 32 rows and keeps their
+//    Q as MFMA B operands in registers for the whole kernel.
+//  * The KV sequence is walked in tiles of 64 keys.  A tile of K and of V (64 x head_dim) is
+//    fetched through the block table with 16-byte coalesced loads, converted to fp16 if the cache
+//    is bf16 / fp8 (fp8: value / per-token scale), and staged in LDS in its natural [key][dim]
+//    layout; LDS is double buffered so the loads of tile t+1 are in flight while tile t is
+//    multiplied.  All four waves read the same tile: every K/V byte is fetched once per 128 rows.
+//  * S^T = K . Q^T (keys x queries) rather than S: in the MFMA result layout a lane then holds 16
+//    keys of ONE query, so the online-softmax row max / row sum are in-lane reductions plus a
+//    single exchange with lane^32, and the fp16 probabilities are already laid out as the B
+//    operand of the next product.
+//  * O^T = V^T . P^T: the A operand needs 8 keys of one head_dim column per lane, i.e. V
+//    transposed.  V stays untransposed in LDS and is read with ds_read_b64_tr_b16, the LDS
+//    transpose load of gfx950 (16 lanes read a 4-key x 16-dim patch and each gets the 4 keys of
+//    its own column).  The two 4-key groups a lane fetches are the keys the S^T layout gives that
+//    lane half, so no shuffle sits between the two products.
+//  * The mask is applied only on tiles that cross the diagonal or the end of the sequence.
 #include "pa_common.hpp"
 #include "pa_host.hpp"
+
+#include <math.h>
+#include <stdio.h>
+
+namespace pa {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr;
+
+// LDS transpose load of gfx950: within each block of 16 lanes, lane i receives element (i % 4)
+// of the 8 bytes addressed by lanes 4j + i/4, j = 0..3 (checked on hardware).
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16* p) {
+  const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)p);
+  return __builtin_bit_cast(half4_t, r);
+}
+
+struct PrefillParams {
+  const void* q;
+  int64_t q_stride;
+  const uint8_t* k;  // paged cache [num_blocks, block_size, kv_heads, D] or dense [tokens, kv_heads, D]
+  const uint8_t* v;
+  const float* k_scale;
+  const float* v_scale;
+  const int32_t* block_tables;  // nullptr = dense K/V indexed by cu_seqlens_k
+  int64_t bt_stride;
+  int64_t kv_token_stride;  // dense mode: elements between consecutive tokens
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  void* out;
+  int64_t out_stride;
+  int q_dtype;
+  int num_q_heads;
+  int num_kv_heads;
+  int bs_log2;
+  int num_blocks;
+  float scale_log2e;
+};
+
+enum : int { SRC_F16 = 0, SRC_BF16 = 1, SRC_FP8 = 2, SRC_F32 = 3 };
+
+constexpr int kBN = 64;  // keys per tile
+
+template <int D>
+struct PrefillLds {
+  static constexpr int KROW = D + 8;   // halfs per K row: +16 bytes keeps 16-byte row reads off one bank
+  static constexpr int VROW = D + 32;  // halfs per V row: +64 bytes spreads the 4-row transpose reads
+  _Float16 k[2][kBN * KROW];
+  _Float16 v[2][kBN * VROW];
+};
+
+// 8 consecutive source elements -> 8 fp16 (fp8: divided by the token's scale)
+template <int SRC>
+__device__ __forceinline__ half8_t load8_as_f16(const uint8_t* p, float inv_scale) {
+  half8_t r;
+  if constexpr (SRC == SRC_F16) {
+    r = *(const half8_t*)p;
+  } else if constexpr (SRC == SRC_BF16) {
+    const uint4 w = *(const uint4*)p;
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      r[2 * i] = (_Float16)__uint_as_float(ww[i] << 16);
+      r[2 * i + 1] = (_Float16)__uint_as_float(ww[i] & 0xffff0000u);
+    }
+  } else if constexpr (SRC == SRC_FP8) {
+    const uint2 w = *(const uint2*)p;
+    const uint32_t ww[2] = {w.x, w.y};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const float2_t lo = fp8x2_to_f32(ww[i], false);
+      const float2_t hi = fp8x2_to_f32(ww[i], true);
+      r[4 * i] = (_Float16)(lo[0] * inv_scale);
+      r[4 * i + 1] = (_Float16)(lo[1] * inv_scale);
+      r[4 * i + 2] = (_Float16)(hi[0] * inv_scale);
+      r[4 * i + 3] = (_Float16)(hi[1] * inv_scale);
+    }
+  } else {
+    const float4 a = *(const float4*)p;
+    const float4 b = *(const float4*)(p + 16);
+    r[0] = (_Float16)a.x; r[1] = (_Float16)a.y; r[2] = (_Float16)a.z; r[3] = (_Float16)a.w;
+    r[4] = (_Float16)b.x; r[5] = (_Float16)b.y; r[6] = (_Float16)b.z; r[7] = (_Float16)b.w;
+  }
+  return r;
+}
+
+template <int SRC>
+constexpr int src_bytes() { return SRC == SRC_FP8 ? 1 : (SRC == SRC_F32 ? 4 : 2); }
+
+template <int D, int HPWG, int SRC>
+__global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams p) {
+  using L = PrefillLds<D>;
+  constexpr int KSTEPS = D / 16;          // MFMA k-steps over head_dim
+  constexpr int MT = D / 32;              // 32-row tiles of O^T
+  constexpr int BM = 128 / HPWG;          // query tokens per workgroup
+  constexpr int CPR = D / 8;              // 8-element chunks per row
+  constexpr int NCH = kBN * CPR / 256;    // chunks per thread per tile (K and V each)
+  constexpr int ES = src_bytes<SRC>();
+  constexpr float NEG_INF = -INFINITY;
+
+  extern __shared__ __align__(16) uint8_t smem_raw[];
+  L& lds = *reinterpret_cast<L*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31;   // query column of this lane
+  const int h = lane >> 5;   // lane half: which 8 of the 16 k-slots
+  const int seq = blockIdx.z;
+  const int q0 = p.cu_q[seq];
+  const int lq = p.cu_q[seq + 1] - q0;
+  const int k0 = p.cu_k[seq];
+  const int lk = p.cu_k[seq + 1] - k0;
+  const int tok0 = blockIdx.x * BM;
+  if (tok0 >= lq) return;
+  const int shift = lk - lq;  // row i sees keys <= i + shift
+
+  const int hslot = (HPWG == 2) ? (wave >> 1) : 0;
+  const int tsub = (HPWG == 2) ? (wave & 1) : wave;
+  const int qhead = blockIdx.y * HPWG + hslot;
+  const int kvh = (blockIdx.y * HPWG) / (p.num_q_heads / p.num_kv_heads);
+  const int tokw0 = tok0 + tsub * 32;            // first token of this wave
+  const int tok = tokw0 + n;                     // this lane's token
+  const bool row_ok = tok < lq;
+  const int qlim = tok + shift;                  // last visible key of this lane's row
+
+  // ---- Q as B operands: [d-step][8 halfs], loaded once ------------------------------------------
+  half8_t qreg[KSTEPS];
+  {
+    const int tq = min(tok, lq - 1);
+    const int64_t base = (int64_t)(q0 + tq) * p.q_stride + (int64_t)qhead * D + 8 * h;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      float x[8];
+      load8_as_f32(p.q, base + ks * 16, p.q_dtype, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qreg[ks][e] = (_Float16)x[e];
+    }
+  }
+
+  float16_t o[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[mt][i] = 0.0f;
+  float m_run = NEG_INF;  // running max of raw scores (same in both lane halves)
+  float l_run = 0.0f;     // running sum of this lane half's probabilities
+
+  // keys the workgroup needs: up to the last valid row's limit
+  const int last_tok = min(tok0 + BM, lq) - 1;
+  const int kend = min(lk, last_tok + shift + 1);
+  const int ntiles = (kend + kBN - 1) / kBN;
+  // this wave's last visible key (wave-uniform)
+  const int wave_last = min(tokw0 + 31, lq - 1) + shift;
+  const bool wave_has_rows = tokw0 < lq;
+
+  const int bs_mask = (1 << p.bs_log2) - 1;
+  const int64_t token_elems = p.block_tables ? (int64_t)p.num_kv_heads * D : p.kv_token_stride;
+  const int32_t* bt_row = p.block_tables ? p.block_tables + seq * p.bt_stride : nullptr;
+  const int bt_last = max((int)p.bt_stride - 1, 0);
+
+  // ---- staging: global -> registers -> LDS ------------------------------------------------------
+  half8_t stage_k[NCH], stage_v[NCH];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int chunk = tid + 256 * c;
+      const int row = chunk / CPR;
+      const int col = chunk % CPR;
+      const int key = t * kBN + row;
+      if (key < lk) {
+        int64_t slot;
+        if (bt_row) {
+          const int blk = min(key >> p.bs_log2, bt_last);
+          const int phys = min(max(bt_row[blk], 0), p.num_blocks - 1);
+          slot = ((int64_t)phys << p.bs_log2) + (key & bs_mask);
+        } else {
+          slot = k0 + key;
+        }
+        const int64_t eoff = slot * token_elems + (int64_t)kvh * D + col * 8;
+        float iks = 1.0f, ivs = 1.0f;
+        if constexpr (SRC == SRC_FP8) {
+          iks = __builtin_amdgcn_rcpf(p.k_scale[slot]);
+          ivs = __builtin_amdgcn_rcpf(p.v_scale[slot]);
+        }
+        stage_k[c] = load8_as_f16<SRC>(p.k + eoff * ES, iks);
+        stage_v[c] = load8_as_f16<SRC>(p.v + eoff * ES, ivs);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          stage_k[c][e] = (_Float16)0.0f;
+          stage_v[c][e] = (_Float16)0.0f;
+        }
+      }
+    }
+  };
+  auto commit = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int chunk = tid + 256 * c;
+      const int row = chunk / CPR;
+      const int col = chunk % CPR;
+      *(half8_t*)&lds.k[buf][row * L::KROW + col * 8] = stage_k[c];
+      *(half8_t*)&lds.v[buf][row * L::VROW + col * 8] = stage_v[c];
+    }
+  };
+
+  // lane-constant parts of the LDS read addresses
+  const int k_lane = n * L::KROW + 8 * h;  // A operand of S^T: key row n, dims 8h.. of a d-step
+  // transpose read: lanes form 4 blocks of 16; block = (dim half of the 32-row tile, lane half);
+  // inside a block lane i supplies the address of key (i/4), dims 4*(i%4).. and receives the 4
+  // keys of dim i
+  const int tr_i = lane & 15;
+  const int tr_dblk = (lane >> 4) & 1;
+  const int v_lane = (4 * h + (tr_i >> 2)) * L::VROW + 16 * tr_dblk + 4 * (tr_i & 3);
+
+  auto compute = [&](int t, int buf) {
+    const int kt0 = t * kBN;
+    // ---- S^T = K . Q^T : two 32-key tiles -------------------------------------------------------
+    float16_t s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * L::KROW + k_lane + ks * 16];
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], s[kt], 0, 0, 0);
+      }
+    }
+    // ---- mask: only tiles that reach past the diagonal of this wave or the sequence end ---------
+    const int wave_first_lim = tokw0 + shift;  // smallest row limit in the wave
+    if (kt0 + kBN - 1 > wave_first_lim || kt0 + kBN > lk) {
+      const int lim = min(qlim, lk - 1);
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kt0 + kt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
+          s[kt][i] = key <= lim ? s[kt][i] : NEG_INF;
+        }
+    }
+    // ---- online softmax over this lane's query column ---------------------------------------------
+    float mloc = s[0][0];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_safe = m_new == NEG_INF ? 0.0f : m_new;
+    const float c = p.scale_log2e;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * c);
+    const float mc = m_safe * c;
+    float psum = 0.0f;
+    half8_t pb[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pr = __builtin_amdgcn_exp2f(fmaf(s[kt][i], c, -mc));
+        psum += pr;
+        pb[kt * 2 + (i >> 3)][i & 7] = (_Float16)pr;
+      }
+    l_run = l_run * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
+    }
+    m_run = m_new;
+    // ---- O^T += V^T . P^T : four 16-key steps x MT row tiles ----------------------------------------
+#pragma unroll
+    for (int k2 = 0; k2 < 4; ++k2) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const _Float16* base = &lds.v[buf][(k2 * 16) * L::VROW + v_lane + 32 * mt];
+        const half4_t lo = lds_read_tr16(base);
+        const half4_t hi = lds_read_tr16(base + 8 * L::VROW);
+        half8_t a;
+        a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
+        a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- tile loop: LDS double buffer, one barrier per tile -------------------------------------------
+  if (ntiles > 0) {
+    fetch(0);
+    commit(0);
+  }
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
+    const bool more = t + 1 < ntiles;
+    if (more) fetch(t + 1);
+    if (wave_has_rows && t * kBN <= wave_last) compute(t, buf);
+    if (more) commit(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- normalise and store ---------------------------------------------------------------------------
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  if (!row_ok) return;
+  const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  const int64_t obase = (int64_t)(q0 + tok) * p.out_stride + (int64_t)qhead * D;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const int d = 32 * mt + 8 * g4 + 4 * h;
+      const float x0 = o[mt][4 * g4] * inv, x1 = o[mt][4 * g4 + 1] * inv;
+      const float x2 = o[mt][4 * g4 + 2] * inv, x3 = o[mt][4 * g4 + 3] * inv;
+      if (p.q_dtype == PA_DTYPE_F32) {
+        *(float4*)((float*)p.out + obase + d) = make_float4(x0, x1, x2, x3);
+      } else if (p.q_dtype == PA_DTYPE_F16) {
+        uint2 w;
+        w.x = (uint32_t)f32_to_f16_bits(x0) | ((uint32_t)f32_to_f16_bits(x1) << 16);
+        w.y = (uint32_t)f32_to_f16_bits(x2) | ((uint32_t)f32_to_f16_bits(x3) << 16);
+        *(uint2*)((uint16_t*)p.out + obase + d) = w;
+      } else {
+        uint2 w;
+        w.x = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
+        w.y = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
+        *(uint2*)((uint16_t*)p.out + obase + d) = w;
+      }
+    }
+}
+
+template <int D, int HPWG, int SRC>
+static int launch_prefill(const PrefillParams& p, dim3 grid, hipStream_t st) {
+  auto kern = paged_prefill_kernel<D, HPWG, SRC>;
+  const size_t smem = sizeof(PrefillLds<D>);
+  static bool attr_set = false;  // per instantiation
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return fail(PA_ERR_LAUNCH, "pa_prefill: cannot raise the dynamic LDS limit");
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, p);
+  return PA_OK;
+}
+
+template <int D, int HPWG>
+static int launch_prefill_src(const PrefillParams& p, dim3 grid, int src, hipStream_t st) {
+  switch (src) {
+    case SRC_F16: return launch_prefill<D, HPWG, SRC_F16>(p, grid, st);
+    case SRC_BF16: return launch_prefill<D, HPWG, SRC_BF16>(p, grid, st);
+    case SRC_FP8: return launch_prefill<D, HPWG, SRC_FP8>(p, grid, st);
+    default: return launch_prefill<D, HPWG, SRC_F32>(p, grid, st);
+  }
+}
+
+}  // namespace pa
 
 using namespace pa;
 
@@ -11,5 +397,82 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
                           int64_t out_token_stride, int64_t num_seqs, int64_t max_seqlen_q,
                           int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                           int64_t block_size, int64_t num_blocks, float scale, void* stream) {
-  return fail(PA_ERR_UNSUPPORTED, "pa_prefill: kernel not built in this revision");
+  if (num_seqs < 0 || max_seqlen_q < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: negative or zero size");
+  if (num_seqs == 0 || max_seqlen_q == 0) return PA_OK;
+  if (!q || !k_cache || !v_cache || !cu_seqlens_q || !cu_seqlens_k || !out)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: null pointer");
+  if (q_dtype != PA_DTYPE_F16 && q_dtype != PA_DTYPE_BF16 && q_dtype != PA_DTYPE_F32)
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill: q_dtype must be f16, bf16 or f32");
+  int src;
+  switch (kv_dtype) {
+    case PA_DTYPE_F16: src = SRC_F16; break;
+    case PA_DTYPE_BF16: src = SRC_BF16; break;
+    case PA_DTYPE_FP8_E4M3: src = SRC_FP8; break;
+    case PA_DTYPE_F32: src = SRC_F32; break;
+    default: return fail(PA_ERR_UNSUPPORTED, "pa_prefill: kv_dtype must be f16, bf16, f32 or fp8-e4m3");
+  }
+  if (src == SRC_FP8 && (!k_scale || !v_scale))
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: fp8 cache needs k_scale and v_scale");
+  if (src == SRC_FP8 && !block_tables)
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill: fp8 K/V need the paged cache (block_tables)");
+  if (head_dim != 64 && head_dim != 128)
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill: head_dim must be 64 or 128");
+  if (num_q_heads % num_kv_heads != 0)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: num_q_heads must be a multiple of num_kv_heads");
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: buffers must be 16-byte aligned");
+  if (q_token_stride < num_q_heads * head_dim || out_token_stride < num_q_heads * head_dim ||
+      q_token_stride % 8 != 0 || out_token_stride % 4 != 0)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: bad q/out token stride");
+  int bs_log2 = 0;
+  int64_t kv_token_stride = 0;
+  if (block_tables) {
+    if (block_size <= 0 || (block_size & (block_size - 1)) != 0)
+      return fail(PA_ERR_UNSUPPORTED, "pa_prefill: block_size must be a power of two");
+    while ((int64_t(1) << bs_log2) < block_size) ++bs_log2;
+    if (num_blocks <= 0 || bt_stride <= 0) return fail(PA_ERR_BAD_ARG, "pa_prefill: bad pool or table size");
+  } else {
+    // dense K/V [total_k_tokens, kv_heads, head_dim]: bt_stride carries the token stride in elements
+    kv_token_stride = bt_stride > 0 ? bt_stride : num_kv_heads * head_dim;
+    if (kv_token_stride < num_kv_heads * head_dim || kv_token_stride % 8 != 0)
+      return fail(PA_ERR_BAD_ARG, "pa_prefill: bad dense K/V token stride");
+    num_blocks = 1;
+  }
+  if (num_seqs > 65535 || num_q_heads > 65535) return fail(PA_ERR_UNSUPPORTED, "pa_prefill: too many sequences or heads");
+
+  const int g = (int)(num_q_heads / num_kv_heads);
+  const int hpwg = (g % 2 == 0) ? 2 : 1;
+  const int bm = 128 / hpwg;
+
+  PrefillParams p;
+  p.q = q;
+  p.q_stride = q_token_stride;
+  p.k = (const uint8_t*)k_cache;
+  p.v = (const uint8_t*)v_cache;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.block_tables = block_tables;
+  p.bt_stride = block_tables ? bt_stride : 0;
+  p.kv_token_stride = kv_token_stride;
+  p.cu_q = cu_seqlens_q;
+  p.cu_k = cu_seqlens_k;
+  p.out = out;
+  p.out_stride = out_token_stride;
+  p.q_dtype = q_dtype;
+  p.num_q_heads = (int)num_q_heads;
+  p.num_kv_heads = (int)num_kv_heads;
+  p.bs_log2 = bs_log2;
+  p.num_blocks = (int)num_blocks;
+  p.scale_log2e = scale * 1.4426950408889634f;
+
+  dim3 grid((unsigned)((max_seqlen_q + bm - 1) / bm), (unsigned)(num_q_heads / hpwg), (unsigned)num_seqs);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (head_dim == 128)
+    rc = hpwg == 2 ? launch_prefill_src<128, 2>(p, grid, src, st) : launch_prefill_src<128, 1>(p, grid, src, st);
+  else
+    rc = hpwg == 2 ? launch_prefill_src<64, 2>(p, grid, src, st) : launch_prefill_src<64, 1>(p, grid, src, st);
+  if (rc != PA_OK) return rc;
+  return check_launch("pa_prefill");
 }

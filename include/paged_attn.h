@@ -172,7 +172,11 @@ int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* cont
  *   cu_seqlens_q/k       [num_seqs + 1] int32 (InferenceContext.cu_seqlens_q / cu_seqlens_k)
  *   block_tables         [num_seqs, bt_stride]; NULL = K/V are dense [total_k_tokens,
  *                        num_kv_heads, head_dim] tensors indexed by cu_seqlens_k (no prefix
- *                        hit: the reference then passes the new k, v themselves)
+ *                        hit: the reference then passes the new k, v themselves) and bt_stride
+ *                        is their token stride in elements (0 = contiguous)
+ *   kv_dtype             PA_DTYPE_F16 / BF16 / F32 / FP8_E4M3 (fp8 only with block_tables);
+ *                        K/V and Q are multiplied as fp16 with fp32 accumulation
+ *   head_dim             64 or 128;  block_size a power of two
  *   max_seqlen_q         upper bound of Lq_s (sizes the launch grid)
  */
 int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
