@@ -20,6 +20,8 @@ from .attention import (
     HAS_FLASH_ATTN,
     HAS_TRITON,
 )
+from .model_runner import ModelRunner, ModelRunnerConfig
+from .qwen3_paged import Qwen3PagedConfig, Qwen3PagedModel
 from . import _native
 
 __all__ = [
@@ -28,4 +30,5 @@ __all__ = [
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",
+    "ModelRunner", "ModelRunnerConfig", "Qwen3PagedConfig", "Qwen3PagedModel",
 ]

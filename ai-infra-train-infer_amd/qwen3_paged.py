@@ -1,0 +1,124 @@
+"""A Qwen3-shaped decoder whose attention layers are PagedAttention modules.
+
+The reference ships no model that owns a PagedAttention (its kv_cache mode drives a
+HuggingFace model and gathers KV in Python, src/inference/model_runner.py:340-433), so this is
+the module a model runner binds caches to (model_runner.py:102-116) and calls as
+`model(input_ids, positions=positions)` (model_runner.py:162).  Block structure follows the
+reference's Qwen3 definition (src/distributed/tensor_parallel.py:307-543): RMSNorm -> q/k/v
+projections -> per-head q/k RMSNorm -> RoPE (half rotation, theta 1e6) -> attention -> o_proj,
+then RMSNorm -> SwiGLU MLP.  GEMMs and norms are plain torch-ROCm ops; only the attention and
+the KV write go through the HIP kernels.  Nothing in forward() synchronises with the host, so a
+decode step can be captured in a HIP graph.
+"""
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .attention import PagedAttention, PartitionedPagedAttention
+from .context import get_context
+
+
+@dataclass
+class Qwen3PagedConfig:
+    """Defaults are the Qwen3-0.6B shape."""
+    vocab_size: int = 151936
+    hidden_size: int = 1024
+    intermediate_size: int = 3072
+    num_layers: int = 28
+    num_heads: int = 16
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    rope_theta: float = 1000000.0
+    rms_norm_eps: float = 1e-6
+    cache_dtype: str = "fp16"
+    partition_size: int = 0        # > 0: use PartitionedPagedAttention with this size
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim, eps):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
+        return (xf * self.weight.float()).to(x.dtype)
+
+
+def apply_rope(x, cos, sin):
+    """x [T, H, D]; cos/sin [T, 1, D] (frequencies repeated over both halves)."""
+    half = x.shape[-1] // 2
+    rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+    return (x.float() * cos + rot.float() * sin).to(x.dtype)
+
+
+class Qwen3PagedLayer(nn.Module):
+    def __init__(self, cfg: Qwen3PagedConfig):
+        super().__init__()
+        self.cfg = cfg
+        q_dim, kv_dim = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.qkv_proj = nn.Linear(cfg.hidden_size, q_dim + 2 * kv_dim, bias=False)
+        self.q_norm = RMSNorm(cfg.head_dim, cfg.rms_norm_eps)
+        self.k_norm = RMSNorm(cfg.head_dim, cfg.rms_norm_eps)
+        if cfg.partition_size > 0:
+            self.attn = PartitionedPagedAttention(cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                                  cfg.cache_dtype, cfg.partition_size)
+        else:
+            self.attn = PagedAttention(cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, cfg.cache_dtype)
+        self.o_proj = nn.Linear(q_dim, cfg.hidden_size, bias=False)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.gate_up_proj = nn.Linear(cfg.hidden_size, 2 * cfg.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
+
+    def forward(self, x, cos, sin):
+        cfg = self.cfg
+        t = x.shape[0]
+        q_dim, kv_dim = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
+        qkv = self.qkv_proj(self.input_layernorm(x))
+        q = qkv[:, :q_dim].view(t, cfg.num_heads, cfg.head_dim)
+        k = qkv[:, q_dim:q_dim + kv_dim].view(t, cfg.num_kv_heads, cfg.head_dim)
+        v = qkv[:, q_dim + kv_dim:].view(t, cfg.num_kv_heads, cfg.head_dim)
+        q = apply_rope(self.q_norm(q), cos, sin)
+        k = apply_rope(self.k_norm(k), cos, sin)
+        a = self.attn(q, k, v)                      # writes k, v into the paged cache, then attends
+        x = x + self.o_proj(a.reshape(t, q_dim))
+        gu = self.gate_up_proj(self.post_attention_layernorm(x))
+        gate, up = gu[:, :cfg.intermediate_size], gu[:, cfg.intermediate_size:]
+        return x + self.down_proj(F.silu(gate) * up)
+
+
+class Qwen3PagedModel(nn.Module):
+    """model(input_ids [T], positions=[T]) -> logits.  Decode: [T, vocab].  Prefill: one row per
+    sequence (its last new token), found from the context's cu_seqlens_q."""
+
+    def __init__(self, cfg: Qwen3PagedConfig):
+        super().__init__()
+        self.cfg = cfg
+        self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size)
+        self.layers = nn.ModuleList(Qwen3PagedLayer(cfg) for _ in range(cfg.num_layers))
+        self.norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False)
+        inv_freq = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32)
+                                             / cfg.head_dim))
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    def rope_tables(self, positions):
+        freqs = positions.float()[:, None] * self.inv_freq[None, :]
+        emb = torch.cat([freqs, freqs], dim=-1)
+        return emb.cos()[:, None, :], emb.sin()[:, None, :]
+
+    def forward(self, input_ids, positions=None):
+        if positions is None:
+            positions = torch.arange(input_ids.shape[0], device=input_ids.device)
+        cos, sin = self.rope_tables(positions)
+        x = self.embed_tokens(input_ids)
+        for layer in self.layers:
+            x = layer(x, cos, sin)
+        ctx = get_context()
+        if ctx.is_prefill and ctx.cu_seqlens_q is not None:
+            x = x[(ctx.cu_seqlens_q[1:] - 1).long()]
+        return self.lm_head(self.norm(x))

@@ -1,0 +1,72 @@
+"""Literal restatement of how the reference's ModelRunner derives the per-step attention
+metadata (TEST INFRASTRUCTURE ONLY; plain Python loops, lists out):
+
+  prefill_metadata   src/inference/model_runner.py:464-540
+  decode_metadata    src/inference/model_runner.py:542-588
+  block_tables       src/inference/model_runner.py:814-828
+
+Pinned by the closed form "slot of position p = block_table[p // BS] * BS + p % BS" in
+tests/test_model_runner_host.py.
+"""
+
+
+def block_tables(sequences):
+    lists = [seq.get("block_table", []) for seq in sequences]
+    if not lists or all(len(bt) == 0 for bt in lists):
+        return None
+    width = max(len(bt) for bt in lists)
+    tables = [[-1] * width for _ in lists]
+    for i, bt in enumerate(lists):
+        for j, block_id in enumerate(bt):
+            tables[i][j] = block_id
+    return tables
+
+
+def prefill_metadata(sequences, block_size):
+    input_ids, positions, slot_mapping = [], [], []
+    cu_q, cu_k = [0], [0]
+    max_q = max_k = 0
+    has_prefix = False
+    for seq in sequences:
+        start = seq["num_cached_tokens"]
+        num_tokens = seq["num_scheduled_tokens"]
+        end = start + num_tokens
+        input_ids.extend(seq["token_ids"][start:end])
+        positions.extend(range(start, end))
+        bt = seq.get("block_table", [])
+        if bt:
+            start_block = start // block_size
+            end_block = (end + block_size - 1) // block_size
+            for i in range(start_block, end_block):
+                slot_start = bt[i] * block_size
+                if i == start_block:
+                    slot_start += start % block_size
+                if i != end_block - 1:
+                    slot_end = bt[i] * block_size + block_size
+                else:
+                    slot_end = bt[i] * block_size + end - i * block_size
+                slot_mapping.extend(range(slot_start, slot_end))
+        cu_q.append(cu_q[-1] + num_tokens)
+        cu_k.append(cu_k[-1] + end)
+        max_q = max(max_q, num_tokens)
+        max_k = max(max_k, end)
+        if start > 0:
+            has_prefix = True
+    return dict(input_ids=input_ids, positions=positions, slot_mapping=slot_mapping or None,
+                cu_seqlens_q=cu_q, cu_seqlens_k=cu_k, max_seqlen_q=max_q, max_seqlen_k=max_k,
+                block_tables=block_tables(sequences) if has_prefix else None)
+
+
+def decode_metadata(sequences, block_size):
+    input_ids, positions, slot_mapping, context_lens = [], [], [], []
+    for seq in sequences:
+        position = len(seq["token_ids"]) - 1
+        last = seq.get("last_block_num_tokens", None)
+        if last is None:
+            last = (position % block_size) + 1
+        input_ids.append(seq["token_ids"][-1])
+        positions.append(position)
+        slot_mapping.append(seq["block_table"][-1] * block_size + last - 1)
+        context_lens.append(len(seq["token_ids"]))
+    return dict(input_ids=input_ids, positions=positions, slot_mapping=slot_mapping,
+                context_lens=context_lens, block_tables=block_tables(sequences))

@@ -1,0 +1,209 @@
+"""The Qwen3-shaped paged model driven by ModelRunner on the GPU: prefill, chunked prefill over a
+cached prefix, decode, HIP-graph replay, and the 28-layer Qwen3-0.6B-shaped decode step."""
+import copy
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import cases
+from oracle import paged_attention_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def dense_reference_logits(model, token_ids):
+    """Last-token logits of one sequence by plain causal attention over all tokens (fp32, CPU,
+    no cache, no paging): the textbook computation the paged path must reproduce."""
+    cfg = model.cfg
+    t = len(token_ids)
+    ids = torch.tensor(token_ids)
+    cos, sin = model.rope_tables(torch.arange(t))
+    x = model.embed_tokens(ids)
+    q_dim, kv_dim = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
+    from ai_infra_train_infer_amd.qwen3_paged import apply_rope
+    for layer in model.layers:
+        qkv = layer.qkv_proj(layer.input_layernorm(x))
+        q = qkv[:, :q_dim].view(t, cfg.num_heads, cfg.head_dim)
+        k = qkv[:, q_dim:q_dim + kv_dim].view(t, cfg.num_kv_heads, cfg.head_dim)
+        v = qkv[:, q_dim + kv_dim:].view(t, cfg.num_kv_heads, cfg.head_dim)
+        q = apply_rope(layer.q_norm(q), cos, sin)
+        k = apply_rope(layer.k_norm(k), cos, sin)
+        rep = cfg.num_heads // cfg.num_kv_heads
+        kk = k.repeat_interleave(rep, dim=1).transpose(0, 1)
+        vv = v.repeat_interleave(rep, dim=1).transpose(0, 1)
+        a = F.scaled_dot_product_attention(q.transpose(0, 1), kk, vv, is_causal=True,
+                                           scale=cfg.head_dim ** -0.5).transpose(0, 1)
+        x = x + layer.o_proj(a.reshape(t, q_dim))
+        gu = layer.gate_up_proj(layer.post_attention_layernorm(x))
+        x = x + layer.down_proj(F.silu(gu[:, :cfg.intermediate_size]) * gu[:, cfg.intermediate_size:])
+    return model.lm_head(model.norm(x[-1:]))[0]
+
+
+def small_model(pa, cache_dtype="fp16", partition_size=0, seed=0):
+    torch.manual_seed(seed)
+    cfg = pa.Qwen3PagedConfig(vocab_size=512, hidden_size=256, intermediate_size=512, num_layers=2,
+                              num_heads=4, num_kv_heads=2, head_dim=64, cache_dtype=cache_dtype,
+                              partition_size=partition_size)
+    return pa.Qwen3PagedModel(cfg).eval()
+
+
+class Session:
+    """Minimal host bookkeeping for the test: a block table per sequence from a free list."""
+
+    def __init__(self, pa, model, gpu, num_blocks=64, cache_dtype="fp16", graphs=None):
+        cfg = model.cfg
+        self.pa, self.bs = pa, 16
+        self.gpu_model = copy.deepcopy(model).half().to(gpu)
+        self.pool = pa.BlockPool(num_blocks, 16, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim,
+                                 dtype=torch.float16, device=gpu, cache_dtype=cache_dtype)
+        self.runner = pa.ModelRunner(self.gpu_model, pa.ModelRunnerConfig(
+            num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
+            head_dim=cfg.head_dim, hidden_size=cfg.hidden_size, vocab_size=cfg.vocab_size, block_size=16,
+            max_num_blocks=16, device="cuda:0", enable_cuda_graph=graphs is not None))
+        self.runner.bind_kv_cache(self.pool.kv_cache_tensor, self.pool.k_scale, self.pool.v_scale,
+                                  self.pool.cache_dtype)
+        if graphs:
+            self.runner.capture_cuda_graphs(graphs)
+        self.free = list(range(num_blocks))[::-1]
+        self.seqs = []
+
+    def add(self, token_ids):
+        self.seqs.append({"token_ids": list(token_ids), "block_table": [], "done": 0})
+
+    def _grow(self, seq, total):
+        while len(seq["block_table"]) * self.bs < total:
+            seq["block_table"].append(self.free.pop())
+
+    def prefill(self, chunk=None):
+        """Schedules the next chunk of every unfinished sequence; returns (logits, their indices)."""
+        batch, who = [], []
+        for i, s in enumerate(self.seqs):
+            left = len(s["token_ids"]) - s["done"]
+            if left == 0:
+                continue
+            n = left if chunk is None else min(chunk, left)
+            self._grow(s, s["done"] + n)
+            batch.append({"token_ids": s["token_ids"], "block_table": s["block_table"],
+                          "num_cached_tokens": s["done"], "num_scheduled_tokens": n})
+            s["done"] += n
+            who.append(i)
+        ids, pos = self.runner.prepare_prefill(batch)
+        return self.runner.run(ids, pos, is_prefill=True), who
+
+    def decode(self, new_tokens):
+        for s, t in zip(self.seqs, new_tokens):
+            s["token_ids"].append(int(t))
+            self._grow(s, len(s["token_ids"]))
+            s["done"] = len(s["token_ids"])
+        ids, pos = self.runner.prepare_decode(self.seqs)
+        return self.runner.run(ids, pos, is_prefill=False)
+
+
+def close(got, want, tol=3e-2):
+    torch.testing.assert_close(got.float().cpu(), want.float(), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("cache_dtype,psize", [("fp16", 0), ("fp16", 32), ("fp8", 0)])
+def test_prefill_then_decode_matches_dense_attention(pa, gpu, cache_dtype, psize):
+    model = small_model(pa, cache_dtype, psize)
+    sess = Session(pa, model, gpu, cache_dtype=cache_dtype)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist() for n in (5, 37, 64, 90)]
+    for p in prompts:
+        sess.add(p)
+    tol = 6e-2 if cache_dtype == "fp8" else 3e-2
+    logits, _ = sess.prefill()
+    ref_model = copy.deepcopy(model).half().float()        # the fp16-rounded weights, fp32 math
+    for i, s in enumerate(sess.seqs):
+        close(logits[i], dense_reference_logits(ref_model, s["token_ids"]), tol)
+    for step in range(3):
+        nxt = torch.randint(0, 512, (4,), generator=g).tolist()
+        logits = sess.decode(nxt)
+        for i, s in enumerate(sess.seqs):
+            close(logits[i], dense_reference_logits(ref_model, s["token_ids"]), tol)
+
+
+def test_chunked_prefill_over_cached_prefix(pa, gpu):
+    model = small_model(pa)
+    sess = Session(pa, model, gpu)
+    g = torch.Generator().manual_seed(2)
+    for n in (70, 33, 128):
+        sess.add(torch.randint(0, 512, (n,), generator=g).tolist())
+    ref_model = copy.deepcopy(model).half().float()
+    final = {}
+    for _ in range(4):                       # 40 tokens per step: later chunks sit on a cached prefix
+        logits, who = sess.prefill(chunk=40)
+        for row, i in enumerate(who):
+            if sess.seqs[i]["done"] == len(sess.seqs[i]["token_ids"]):
+                final[i] = logits[row].clone()
+    assert pa.get_context().block_tables is None            # run() reset the context
+    assert sorted(final) == [0, 1, 2]
+    for i, s in enumerate(sess.seqs):
+        close(final[i], dense_reference_logits(ref_model, s["token_ids"]))
+
+
+def test_graph_replay_equals_eager_on_every_replay(pa, gpu):
+    model = small_model(pa, seed=3)
+    eager = Session(pa, model, gpu)
+    graph = Session(pa, model, gpu, graphs=[2, 4])
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist() for n in (9, 40, 17)]
+    for p in prompts:
+        eager.add(p)
+        graph.add(p)
+    close(graph.prefill()[0], eager.prefill()[0].cpu(), 1e-3)
+    for step in range(5):                    # 3 sequences replay the batch-4 graph with one padded row
+        nxt = torch.randint(0, 512, (3,), generator=g).tolist()
+        le = eager.decode(nxt)
+        lg = graph.decode(nxt)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(lg.float().cpu(), le.float().cpu(), rtol=2e-3, atol=2e-3)
+        # the caches the two sessions wrote are identical too
+        assert torch.equal(graph.pool.kv_cache_tensor[:, :, graph.seqs[1]["block_table"][0]].cpu(),
+                           eager.pool.kv_cache_tensor[:, :, eager.seqs[1]["block_table"][0]].cpu())
+        # eager work between replays
+        _ = (le.float() @ le.float().t()).sum().item()
+
+
+def test_config5b_qwen3_0p6b_shaped_decode_step(pa, gpu):
+    """28 layers, hidden 1024, 16q/8kv x 128, random init, batch 64 at context 2048: one decode
+    step; the attention of four layers is checked against the oracle on the pool they used."""
+    torch.manual_seed(5)
+    cfg = pa.Qwen3PagedConfig()
+    with torch.device(gpu):
+        model = pa.Qwen3PagedModel(cfg).half().eval()
+    B, CTX, BS = 64, 2048, 16
+    nb = B * (CTX // BS) + 64
+    pool = pa.BlockPool(nb, BS, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim, dtype=torch.float16, device=gpu)
+    g = torch.Generator(device=gpu).manual_seed(6)
+    kv = pool.kv_cache_tensor
+    for l in range(cfg.num_layers):          # history: N(0,1) keys and values
+        kv[0, l].copy_(torch.randn(kv[0, l].shape, generator=g, device=gpu, dtype=torch.float32))
+        kv[1, l].copy_(torch.randn(kv[1, l].shape, generator=g, device=gpu, dtype=torch.float32))
+    runner = pa.ModelRunner(model, pa.ModelRunnerConfig(
+        num_layers=28, num_heads=16, num_kv_heads=8, head_dim=128, hidden_size=1024, block_size=BS,
+        max_num_blocks=CTX // BS, device="cuda:0", enable_cuda_graph=False))
+    runner.bind_kv_cache(kv)
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(7))[:B * (CTX // BS)].view(B, -1)
+    seqs = [{"token_ids": [1] * CTX, "block_table": perm[b].tolist()} for b in range(B)]
+    grabbed = {}
+    check_layers = (0, 9, 27)
+    hooks = []
+    for l in check_layers:
+        def hook(mod, args, out, l=l):
+            grabbed[l] = (args[0].detach().clone(), out.detach().clone())
+        hooks.append(model.layers[l].attn.register_forward_hook(hook))
+    ids, pos = runner.prepare_decode(seqs)
+    tables = pa.get_context().block_tables.cpu()
+    lens = pa.get_context().context_lens.cpu()
+    logits = runner.run(ids, pos, is_prefill=False)
+    torch.cuda.synchronize()
+    for h in hooks:
+        h.remove()
+    assert tuple(logits.shape) == (B, cfg.vocab_size) and torch.isfinite(logits).all()
+    for l in check_layers:
+        q, out = grabbed[l]
+        want = oracle.decode(q.cpu(), kv[0, l].cpu(), kv[1, l].cpu(), tables, lens, cfg.head_dim ** -0.5)
+        torch.testing.assert_close(out.cpu().float(), want.float(), rtol=1e-3, atol=2e-3)
