@@ -74,12 +74,14 @@ enum : int { SRC_F16 = 0, SRC_BF16 = 1, SRC_FP8 = 2, SRC_F32 = 3 };
 
 constexpr int kBN = 64;  // keys per tile
 
+// One stage of a K or V tile in LDS: [key][head_dim] fp16 rows with no padding; the 16-byte
+// chunk c of row r lives at chunk position c ^ (r & (CPR-1)) (CPR = chunks per row), so that the
+// 16 lanes that read the same chunk index of 16 consecutive rows (the MFMA A-operand reads of K)
+// and the 4-row x 32-byte patches of the transpose reads of V all fall on distinct banks.
 template <int D>
 struct PrefillLds {
-  static constexpr int KROW = D + 8;   // halfs per K row: +16 bytes keeps 16-byte row reads off one bank
-  static constexpr int VROW = D + 32;  // halfs per V row: +64 bytes spreads the 4-row transpose reads
-  _Float16 k[2][kBN * KROW];
-  _Float16 v[2][kBN * VROW];
+  _Float16 k[2][kBN * D];
+  _Float16 v[2][kBN * D];
 };
 
 // 8 consecutive source elements -> 8 fp16 (fp8: divided by the token's scale)
@@ -120,9 +122,12 @@ __device__ __forceinline__ half8_t load8_as_f16(const uint8_t* p, float inv_scal
 template <int SRC>
 constexpr int src_bytes() { return SRC == SRC_FP8 ? 1 : (SRC == SRC_F32 ? 4 : 2); }
 
+// DIRECT: fp16 sources go global -> LDS with global_load_lds_dwordx4 (no staging registers, two
+// workgroups per CU); other source types are converted in registers on the way (one per CU).
 template <int D, int HPWG, int SRC>
-__global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_kernel(const PrefillParams p) {
   using L = PrefillLds<D>;
+  constexpr bool DIRECT = SRC == SRC_F16;
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over head_dim
   constexpr int MT = D / 32;              // 32-row tiles of O^T
   constexpr int BM = 128 / HPWG;          // query tokens per workgroup
@@ -192,25 +197,38 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams 
   const int32_t* bt_row = p.block_tables ? p.block_tables + seq * p.bt_stride : nullptr;
   const int bt_last = max((int)p.bt_stride - 1, 0);
 
-  // ---- staging: global -> registers -> LDS ------------------------------------------------------
-  half8_t stage_k[NCH], stage_v[NCH];
-  auto fetch = [&](int t) {
+  // ---- staging: global -> (registers ->) LDS ---------------------------------------------------------
+  // chunk = 16 bytes of fp16 = 8 head-dim elements; thread `tid` moves chunks tid, tid+256, ...
+  // i.e. one instruction of a wave covers 64 / CPR whole rows, contiguous in LDS.
+  constexpr int SWZ = CPR - 1;
+  auto row_slot = [&](int key) -> int64_t {   // physical row of a key (clamped: never faults)
+    const int kk = min(key, lk - 1);
+    if (bt_row) {
+      const int blk = min(kk >> p.bs_log2, bt_last);
+      const int phys = min(max(bt_row[blk], 0), p.num_blocks - 1);
+      return ((int64_t)phys << p.bs_log2) + (kk & bs_mask);
+    }
+    return (int64_t)k0 + kk;
+  };
+  half8_t stage_k[DIRECT ? 1 : NCH], stage_v[DIRECT ? 1 : NCH];
+  auto fetch = [&](int t, int buf) {
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int chunk = tid + 256 * c;
       const int row = chunk / CPR;
-      const int col = chunk % CPR;
+      const int pos = chunk % CPR;                 // chunk position inside the LDS row
+      const int col = pos ^ (row & SWZ);           // head-dim chunk that belongs there
       const int key = t * kBN + row;
-      if (key < lk) {
-        int64_t slot;
-        if (bt_row) {
-          const int blk = min(key >> p.bs_log2, bt_last);
-          const int phys = min(max(bt_row[blk], 0), p.num_blocks - 1);
-          slot = ((int64_t)phys << p.bs_log2) + (key & bs_mask);
-        } else {
-          slot = k0 + key;
-        }
-        const int64_t eoff = slot * token_elems + (int64_t)kvh * D + col * 8;
+      const int64_t slot = row_slot(key);          // rows past the sequence end re-read its last row (masked later)
+      const int64_t eoff = slot * token_elems + (int64_t)kvh * D + col * 8;
+      if constexpr (DIRECT) {
+        // LDS destination = wave-uniform base + lane * 16 bytes
+        const int wbase = (256 * c + (tid & ~63)) * 8;   // in halfs
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.k + eoff * ES),
+                                         (__attribute__((address_space(3))) void*)&lds.k[buf][wbase], 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.v + eoff * ES),
+                                         (__attribute__((address_space(3))) void*)&lds.v[buf][wbase], 16, 0, 0);
+      } else {
         float iks = 1.0f, ivs = 1.0f;
         if constexpr (SRC == SRC_FP8) {
           iks = __builtin_amdgcn_rcpf(p.k_scale[slot]);
@@ -218,34 +236,40 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams 
         }
         stage_k[c] = load8_as_f16<SRC>(p.k + eoff * ES, iks);
         stage_v[c] = load8_as_f16<SRC>(p.v + eoff * ES, ivs);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          stage_k[c][e] = (_Float16)0.0f;
-          stage_v[c][e] = (_Float16)0.0f;
-        }
       }
     }
   };
   auto commit = [&](int buf) {
+    if constexpr (!DIRECT) {
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int chunk = tid + 256 * c;
-      const int row = chunk / CPR;
-      const int col = chunk % CPR;
-      *(half8_t*)&lds.k[buf][row * L::KROW + col * 8] = stage_k[c];
-      *(half8_t*)&lds.v[buf][row * L::VROW + col * 8] = stage_v[c];
+      for (int c = 0; c < NCH; ++c) {
+        const int chunk = tid + 256 * c;
+        *(half8_t*)&lds.k[buf][chunk * 8] = stage_k[c];
+        *(half8_t*)&lds.v[buf][chunk * 8] = stage_v[c];
+      }
     }
   };
 
-  // lane-constant parts of the LDS read addresses
-  const int k_lane = n * L::KROW + 8 * h;  // A operand of S^T: key row n, dims 8h.. of a d-step
-  // transpose read: lanes form 4 blocks of 16; block = (dim half of the 32-row tile, lane half);
-  // inside a block lane i supplies the address of key (i/4), dims 4*(i%4).. and receives the 4
-  // keys of dim i
+  // ---- loop-invariant LDS read offsets (in halfs, before the buffer / tile-row offsets) ------------
+  // S^T A operand: key row n of a 32-key tile, head-dim chunk 2*ks + h
+  int k_off[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = n * D + (((2 * ks + h) ^ (n & SWZ)) << 3);
+  // O^T A operand through the transpose read: lanes form 4 blocks of 16 = (dim half of the
+  // 32-row tile, lane half); inside a block lane i supplies the address of key (i/4), dims
+  // 4*(i%4).. and receives the 4 keys of dim i.  lo/hi = the two 4-key groups of a 16-key step
+  // that the S^T result layout gives this lane half: keys 4h.. and 8+4h..
   const int tr_i = lane & 15;
   const int tr_dblk = (lane >> 4) & 1;
-  const int v_lane = (4 * h + (tr_i >> 2)) * L::VROW + 16 * tr_dblk + 4 * (tr_i & 3);
+  int v_off[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int row = 8 * r + 4 * h + (tr_i >> 2);                     // row & 15 of the key
+      const int chunk = 4 * mt + 2 * tr_dblk + ((tr_i & 3) >> 1);      // head-dim chunk
+      v_off[mt][r] = row * D + ((chunk ^ (row & SWZ)) << 3) + 4 * (tr_i & 1);
+    }
 
   auto compute = [&](int t, int buf) {
     const int kt0 = t * kBN;
@@ -257,7 +281,7 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams 
       for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * L::KROW + k_lane + ks * 16];
+        const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * D + k_off[ks]];
         s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], s[kt], 0, 0, 0);
       }
     }
@@ -308,9 +332,8 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams 
     for (int k2 = 0; k2 < 4; ++k2) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const _Float16* base = &lds.v[buf][(k2 * 16) * L::VROW + v_lane + 32 * mt];
-        const half4_t lo = lds_read_tr16(base);
-        const half4_t hi = lds_read_tr16(base + 8 * L::VROW);
+        const half4_t lo = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][0]]);
+        const half4_t hi = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][1]]);
         half8_t a;
         a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
         a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
@@ -321,17 +344,17 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(const PrefillParams 
 
   // ---- tile loop: LDS double buffer, one barrier per tile -------------------------------------------
   if (ntiles > 0) {
-    fetch(0);
+    fetch(0, 0);
     commit(0);
   }
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const int buf = t & 1;
     const bool more = t + 1 < ntiles;
-    if (more) fetch(t + 1);
+    if (more) fetch(t + 1, buf ^ 1);   // direct loads land in the other buffer while this one is used
     if (wave_has_rows && t * kBN <= wave_last) compute(t, buf);
     if (more) commit(buf ^ 1);
-    __syncthreads();
+    __syncthreads();                   // also waits for this wave's outstanding loads into LDS
   }
 
   // ---- normalise and store ---------------------------------------------------------------------------

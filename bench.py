@@ -105,6 +105,33 @@ def cpu_baseline(torch, w, scale, sample_seqs, bs, repeats=3):
     return best, out
 
 
+def prefill_cfg5a(pa, torch, dev, steps, warmup):
+    """BASELINE configs[4], first half: 8 sequences x (2048 cached + 512 new tokens), bf16 Q, FP16
+    KV, causal within the chunk; judged against the dense fp16 MFMA peak."""
+    S, CACHED, NEW, HQ, HKV, D, BS = 8, 2048, 512, 16, 8, 128, 16
+    g = torch.Generator(device=dev).manual_seed(1005)
+    bps = (CACHED + NEW) // BS
+    nb = S * bps + 32
+    tables = torch.randperm(nb, generator=g, device=dev)[:S * bps].view(S, bps).to(torch.int32).contiguous()
+    kc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+    vc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+    q = torch.randn(S * NEW, HQ, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    cu_q = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * NEW
+    cu_k = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * (CACHED + NEW)
+    out = torch.empty_like(q)
+
+    def step():
+        pa.paged_prefill(q, kc, vc, cu_q, cu_k, NEW, D ** -0.5, block_tables=tables, out=out)
+
+    ms, _ = time_steps(torch, step, steps, warmup)
+    pairs = NEW * CACHED + NEW * (NEW + 1) // 2            # visible (query, key) pairs per head
+    flops = pairs * D * 2 * 2 * HQ * S                     # QK^T and PV, 2 flops per MAC
+    return {"workload": "8 x (2048 cached + 512 new), 16q/8kv, d128, bf16 Q, FP16 KV",
+            "us": round(ms * 1e3, 1), "gflop": round(flops / 1e9, 2),
+            "tflops": round(flops / ms / 1e9, 1), "peak_tflops": 2500.0,
+            "frac_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -114,6 +141,9 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=8)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 1 GiB device-to-device copies (known traffic: 1 GiB read, "
+                         "1 GiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures the single-GPU hot path only; --gpus %d is not "
@@ -127,6 +157,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     B, CTX, HQ, HKV, D, BS = args.batch, args.ctx, 16, 8, 128, 16
     scale = 1.0 / math.sqrt(D)
@@ -185,6 +224,7 @@ def main():
         del w
         torch.cuda.empty_cache()
 
+    prefill = prefill_cfg5a(pa, torch, dev, max(10, args.steps // 4), max(2, args.warmup // 4))
     f16, f8 = results["fp16"], results["fp8"]
     line = {
         "metric": "paged decode attn achieved HBM GB/s (% peak) + us/step at bs=64 ctx=4k",
@@ -227,6 +267,7 @@ def main():
             "traffic": None,
         },
     }
+    line["prefill_mfma"] = prefill
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
