@@ -75,9 +75,16 @@ enum : int { SRC_F16 = 0, SRC_BF16 = 1, SRC_FP8 = 2, SRC_F32 = 3 };
 constexpr int kBN = 64;  // keys per tile
 
 // One stage of a K or V tile in LDS: [key][head_dim] fp16 rows with no padding; the 16-byte
-// chunk c of row r lives at chunk position c ^ (r & (CPR-1)) (CPR = chunks per row), so that the
-// 16 lanes that read the same chunk index of 16 consecutive rows (the MFMA A-operand reads of K)
-// and the 4-row x 32-byte patches of the transpose reads of V all fall on distinct banks.
+// chunk c of row r lives at chunk position c ^ swz(r).  swz swaps the two low bit pairs of the
+// row number, so that (a) 16 consecutive rows get 16 different values: the 16 lanes that read
+// the same chunk index of 16 rows (MFMA A-operand reads of K) hit distinct banks, and (b) 4
+// consecutive rows differ in bits 2..3: the 4-row x 64-byte patch that 32 lanes fetch in one
+// pass of a transpose read of V spreads over 16 distinct chunk positions.
+template <int CPR>
+__device__ __forceinline__ constexpr int swz(int row) {
+  return (((row & 3) << 2) | ((row >> 2) & 3)) & (CPR - 1);
+}
+
 template <int D>
 struct PrefillLds {
   _Float16 k[2][kBN * D];
@@ -200,7 +207,6 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   // ---- staging: global -> (registers ->) LDS ---------------------------------------------------------
   // chunk = 16 bytes of fp16 = 8 head-dim elements; thread `tid` moves chunks tid, tid+256, ...
   // i.e. one instruction of a wave covers 64 / CPR whole rows, contiguous in LDS.
-  constexpr int SWZ = CPR - 1;
   auto row_slot = [&](int key) -> int64_t {   // physical row of a key (clamped: never faults)
     const int kk = min(key, lk - 1);
     if (bt_row) {
@@ -211,32 +217,63 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     return (int64_t)k0 + kk;
   };
   half8_t stage_k[DIRECT ? 1 : NCH], stage_v[DIRECT ? 1 : NCH];
+  // Fast path for tiles that lie wholly inside the sequence: the 64/CPR rows one wave moves per
+  // instruction belong to one block (block_size >= 16) or are consecutive dense rows, so the
+  // row base is wave-uniform (scalar table load, scalar 64-bit base) and the per-lane part of
+  // the address never changes between tiles.
+  const bool uniform_rows = bt_row == nullptr || p.bs_log2 >= 4;
+  uint32_t lane_part[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int chunk = tid + 256 * c;
+    const int row = chunk / CPR;
+    const int col = (chunk % CPR) ^ swz<CPR>(row);
+    lane_part[c] = (uint32_t)(((lane / CPR) * token_elems + (int64_t)kvh * D + col * 8) * ES);
+  }
+  auto move_chunk = [&](int c, int buf, const uint8_t* kp, const uint8_t* vp, int64_t slot) {
+    if constexpr (DIRECT) {
+      const int wbase = (256 * c + (tid & ~63)) * 8;   // LDS destination = wave base + lane * 16 bytes
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
+                                       (__attribute__((address_space(3))) void*)&lds.k[buf][wbase], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
+                                       (__attribute__((address_space(3))) void*)&lds.v[buf][wbase], 16, 0, 0);
+    } else {
+      float iks = 1.0f, ivs = 1.0f;
+      if constexpr (SRC == SRC_FP8) {
+        iks = __builtin_amdgcn_rcpf(p.k_scale[slot]);
+        ivs = __builtin_amdgcn_rcpf(p.v_scale[slot]);
+      }
+      stage_k[c] = load8_as_f16<SRC>(kp, iks);
+      stage_v[c] = load8_as_f16<SRC>(vp, ivs);
+    }
+  };
   auto fetch = [&](int t, int buf) {
+    if (uniform_rows && (t + 1) * kBN <= lk) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int row0 = (256 * c + 64 * wave) / CPR;      // first row of this wave's instruction
+        const int key0 = t * kBN + row0;
+        int64_t slot0;
+        if (bt_row) {
+          const int blk = min(key0 >> p.bs_log2, bt_last);
+          const int phys = min(max(bt_row[blk], 0), p.num_blocks - 1);
+          slot0 = ((int64_t)phys << p.bs_log2) + (key0 & bs_mask);
+        } else {
+          slot0 = (int64_t)k0 + key0;
+        }
+        const int64_t base = slot0 * token_elems * ES;
+        move_chunk(c, buf, p.k + base + lane_part[c], p.v + base + lane_part[c], slot0 + lane / CPR);
+      }
+      return;
+    }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
       const int chunk = tid + 256 * c;
       const int row = chunk / CPR;
-      const int pos = chunk % CPR;                 // chunk position inside the LDS row
-      const int col = pos ^ (row & SWZ);           // head-dim chunk that belongs there
-      const int key = t * kBN + row;
-      const int64_t slot = row_slot(key);          // rows past the sequence end re-read its last row (masked later)
-      const int64_t eoff = slot * token_elems + (int64_t)kvh * D + col * 8;
-      if constexpr (DIRECT) {
-        // LDS destination = wave-uniform base + lane * 16 bytes
-        const int wbase = (256 * c + (tid & ~63)) * 8;   // in halfs
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.k + eoff * ES),
-                                         (__attribute__((address_space(3))) void*)&lds.k[buf][wbase], 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.v + eoff * ES),
-                                         (__attribute__((address_space(3))) void*)&lds.v[buf][wbase], 16, 0, 0);
-      } else {
-        float iks = 1.0f, ivs = 1.0f;
-        if constexpr (SRC == SRC_FP8) {
-          iks = __builtin_amdgcn_rcpf(p.k_scale[slot]);
-          ivs = __builtin_amdgcn_rcpf(p.v_scale[slot]);
-        }
-        stage_k[c] = load8_as_f16<SRC>(p.k + eoff * ES, iks);
-        stage_v[c] = load8_as_f16<SRC>(p.v + eoff * ES, ivs);
-      }
+      const int col = (chunk % CPR) ^ swz<CPR>(row);   // head-dim chunk that belongs at this LDS position
+      const int64_t slot = row_slot(t * kBN + row);    // rows past the sequence end re-read its last row (masked later)
+      const int64_t eoff = (slot * token_elems + (int64_t)kvh * D + col * 8) * ES;
+      move_chunk(c, buf, p.k + eoff, p.v + eoff, slot);
     }
   };
   auto commit = [&](int buf) {
@@ -254,7 +291,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   // S^T A operand: key row n of a 32-key tile, head-dim chunk 2*ks + h
   int k_off[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = n * D + (((2 * ks + h) ^ (n & SWZ)) << 3);
+  for (int ks = 0; ks < KSTEPS; ++ks) k_off[ks] = n * D + (((2 * ks + h) ^ swz<CPR>(n)) << 3);
   // O^T A operand through the transpose read: lanes form 4 blocks of 16 = (dim half of the
   // 32-row tile, lane half); inside a block lane i supplies the address of key (i/4), dims
   // 4*(i%4).. and receives the 4 keys of dim i.  lo/hi = the two 4-key groups of a 16-key step
@@ -268,7 +305,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     for (int r = 0; r < 2; ++r) {
       const int row = 8 * r + 4 * h + (tr_i >> 2);                     // row & 15 of the key
       const int chunk = 4 * mt + 2 * tr_dblk + ((tr_i & 3) >> 1);      // head-dim chunk
-      v_off[mt][r] = row * D + ((chunk ^ (row & SWZ)) << 3) + 4 * (tr_i & 1);
+      v_off[mt][r] = row * D + ((chunk ^ swz<CPR>(row)) << 3) + 4 * (tr_i & 1);
     }
 
   auto compute = [&](int t, int buf) {
