@@ -33,6 +33,8 @@
 #include <math.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 namespace pa {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -156,14 +158,17 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   const int lq = p.cu_q[seq + 1] - q0;
   const int k0 = p.cu_k[seq];
   const int lk = p.cu_k[seq + 1] - k0;
-  const int tok0 = blockIdx.x * BM;
+  // blockIdx.x (fastest, dealt round-robin to the 8 XCDs) is the head group: all query tiles of
+  // one KV head then run on the same XCD and share its L2, so a K/V tile is fetched from HBM
+  // once instead of once per query tile.
+  const int tok0 = blockIdx.y * BM;
   if (tok0 >= lq) return;
   const int shift = lk - lq;  // row i sees keys <= i + shift
 
   const int hslot = (HPWG == 2) ? (wave >> 1) : 0;
   const int tsub = (HPWG == 2) ? (wave & 1) : wave;
-  const int qhead = blockIdx.y * HPWG + hslot;
-  const int kvh = (blockIdx.y * HPWG) / (p.num_q_heads / p.num_kv_heads);
+  const int qhead = blockIdx.x * HPWG + hslot;
+  const int kvh = (blockIdx.x * HPWG) / (p.num_q_heads / p.num_kv_heads);
   const int tokw0 = tok0 + tsub * 32;            // first token of this wave
   const int tok = tokw0 + n;                     // this lane's token
   const bool row_ok = tok < lq;
@@ -308,7 +313,10 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
       v_off[mt][r] = row * D + ((chunk ^ swz<CPR>(row)) << 3) + 4 * (tr_i & 1);
     }
 
-  auto compute = [&](int t, int buf) {
+  // `buf` is a compile-time constant (the tile loop is unrolled by two) so that every LDS read
+  // below is "loop-invariant register + immediate offset".
+  auto compute = [&](int t, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
     const int kt0 = t * kBN;
     // ---- S^T = K . Q^T : two 32-key tiles -------------------------------------------------------
     float16_t s[2];
@@ -341,11 +349,24 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
 #pragma unroll
       for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m_run, mloc);
-    const float m_safe = m_new == NEG_INF ? 0.0f : m_new;
+    // Lazy rescale: the running max only follows the true max when it has grown by more than
+    // 2^8 in the exponent domain, so probabilities stay <= 256 (exact enough in fp16 and fp32)
+    // and the 64-register rescale of O^T runs on the first tile and then almost never.  The
+    // final division by the row sum removes whatever reference point was used.
     const float c = p.scale_log2e;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * c);
-    const float mc = m_safe * c;
+    const bool grow = (mloc - m_run) * c > 8.0f;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(grow) != 0, 0)) {
+      const float m_new = grow ? mloc : m_run;
+      // exp2(-inf) = 0 on a row's first visible tile; rows that do not move keep factor 1
+      const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * c) : 1.0f;
+      l_run *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
+      m_run = m_new;
+    }
+    const float mc = (m_run == NEG_INF ? 0.0f : m_run) * c;
     float psum = 0.0f;
     half8_t pb[4];
 #pragma unroll
@@ -356,14 +377,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
         psum += pr;
         pb[kt * 2 + (i >> 3)][i & 7] = (_Float16)pr;
       }
-    l_run = l_run * alpha + psum;
-    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
-    }
-    m_run = m_new;
+    l_run += psum;
     // ---- O^T += V^T . P^T : four 16-key steps x MT row tiles ----------------------------------------
 #pragma unroll
     for (int k2 = 0; k2 < 4; ++k2) {
@@ -385,13 +399,17 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     commit(0);
   }
   __syncthreads();
-  for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
+  auto step = [&](int t, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
     const bool more = t + 1 < ntiles;
     if (more) fetch(t + 1, buf ^ 1);   // direct loads land in the other buffer while this one is used
-    if (wave_has_rows && t * kBN <= wave_last) compute(t, buf);
+    if (wave_has_rows && t * kBN <= wave_last) compute(t, buf_tag);
     if (more) commit(buf ^ 1);
     __syncthreads();                   // also waits for this wave's outstanding loads into LDS
+  };
+  for (int t = 0; t < ntiles; t += 2) {
+    step(t, std::integral_constant<int, 0>{});
+    if (t + 1 < ntiles) step(t + 1, std::integral_constant<int, 1>{});
   }
 
   // ---- normalise and store ---------------------------------------------------------------------------
@@ -499,7 +517,8 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
       return fail(PA_ERR_BAD_ARG, "pa_prefill: bad dense K/V token stride");
     num_blocks = 1;
   }
-  if (num_seqs > 65535 || num_q_heads > 65535) return fail(PA_ERR_UNSUPPORTED, "pa_prefill: too many sequences or heads");
+  if (num_seqs > 65535 || max_seqlen_q > 65535 * 64)
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill: too many sequences or query tokens for one launch");
 
   const int g = (int)(num_q_heads / num_kv_heads);
   const int hpwg = (g % 2 == 0) ? 2 : 1;
@@ -526,7 +545,7 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
   p.num_blocks = (int)num_blocks;
   p.scale_log2e = scale * 1.4426950408889634f;
 
-  dim3 grid((unsigned)((max_seqlen_q + bm - 1) / bm), (unsigned)(num_q_heads / hpwg), (unsigned)num_seqs);
+  dim3 grid((unsigned)(num_q_heads / hpwg), (unsigned)((max_seqlen_q + bm - 1) / bm), (unsigned)num_seqs);
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (head_dim == 128)
