@@ -252,7 +252,14 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
       stage_v[c] = load8_as_f16<SRC>(vp, ivs);
     }
   };
-  auto fetch = [&](int t, int buf) {
+  // Block-table entries of a tile, fetched one tile ahead of the loads that need them so that no
+  // load ever waits on another: lane l holds the entry of chunk group l % NCH of this wave.
+  auto load_ids = [&](int t) -> int {
+    if (!bt_row) return 0;
+    const int row0 = (256 * (lane % NCH) + 64 * wave) / CPR;
+    return bt_row[min((t * kBN + row0) >> p.bs_log2, bt_last)];
+  };
+  auto fetch = [&](int t, int buf, int ids) {
     if (uniform_rows && (t + 1) * kBN <= lk) {
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
@@ -260,8 +267,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
         const int key0 = t * kBN + row0;
         int64_t slot0;
         if (bt_row) {
-          const int blk = min(key0 >> p.bs_log2, bt_last);
-          const int phys = min(max(bt_row[blk], 0), p.num_blocks - 1);
+          const int phys = min(max(__builtin_amdgcn_readlane(ids, c), 0), p.num_blocks - 1);
           slot0 = ((int64_t)phys << p.bs_log2) + (key0 & bs_mask);
         } else {
           slot0 = (int64_t)k0 + key0;
@@ -394,17 +400,22 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   };
 
   // ---- tile loop: LDS double buffer, one barrier per tile -------------------------------------------
+  int ids = 0;
   if (ntiles > 0) {
-    fetch(0, 0);
+    ids = load_ids(0);
+    fetch(0, 0, ids);
     commit(0);
+    if (ntiles > 1) ids = load_ids(1);
   }
   __syncthreads();
   auto step = [&](int t, auto buf_tag) {
     constexpr int buf = decltype(buf_tag)::value;
-    const bool more = t + 1 < ntiles;
-    if (more) fetch(t + 1, buf ^ 1);   // direct loads land in the other buffer while this one is used
+    if (t + 1 < ntiles) {
+      fetch(t + 1, buf ^ 1, ids);      // direct loads land in the other buffer while this one is used
+      if (t + 2 < ntiles) ids = load_ids(t + 2);
+    }
     if (wave_has_rows && t * kBN <= wave_last) compute(t, buf_tag);
-    if (more) commit(buf ^ 1);
+    if (t + 1 < ntiles) commit(buf ^ 1);
     __syncthreads();                   // also waits for this wave's outstanding loads into LDS
   };
   for (int t = 0; t < ntiles; t += 2) {
