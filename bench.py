@@ -65,6 +65,21 @@ def build_workload(pa, torch, dev, batch, ctx, hq, hkv, d, bs, fp8, seed):
                 block_tables=tables, context_lens=lens, num_blocks=nb)
 
 
+def measured_traffic(key):
+    """HBM bytes per launch of the decode kernel as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE (scaled by a plain copy of known size); read from the committed summary of those
+    runs, None if it is absent.  Counters cannot be sampled from inside this process."""
+    path = os.path.join(ROOT, "profiles", "paged_decode_bs64_ctx4096_pmc_traffic.txt")
+    try:
+        with open(path) as f:
+            for ln in f:
+                if ln.startswith(key + " ="):
+                    return int(ln.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def time_steps(torch, fn, steps, warmup):
     """W untimed + K timed calls on the current stream; returns (ms per step by HIP events,
     ms per step by the host clock around synchronised ends)."""
@@ -264,7 +279,8 @@ def main():
             "frac": round(f16["kernel_gbps"] / HBM_PEAK_GBPS, 4),
             "kernel_us": round(f16["kernel_us"], 2),
             "algorithmic_bytes": f16["bytes"],
-            "traffic": None,
+            "traffic": measured_traffic("traffic_bytes_fp16") if (B, CTX) == (64, 4096) else None,
+            "traffic_source": "profiles/paged_decode_bs64_ctx4096_pmc_traffic.txt (rocprofv3 --pmc, copy-calibrated)",
         },
     }
     line["prefill_mfma"] = prefill
