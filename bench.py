@@ -147,6 +147,28 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup):
             "frac_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
 
 
+def kv_store_times(pa, torch, dev, steps, warmup):
+    """Paged KV-cache write of one decode step (64 new tokens) and of one prefill chunk (4096
+    tokens), FP16 copy and FP8 quantising store.  Latency-bound: reported in microseconds only."""
+    HKV, D, BS, NB = 8, 128, 16, 4096 // 16 + 64
+    g = torch.Generator(device=dev).manual_seed(7)
+    out = {}
+    for n in (64, 4096):
+        k = torch.randn(n, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+        v = torch.randn(n, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+        slots = torch.randperm(NB * BS, generator=g, device=dev)[:n].to(torch.int32)
+        kc = torch.zeros(NB, BS, HKV, D, dtype=torch.float16, device=dev)
+        vc = torch.zeros_like(kc)
+        k8 = torch.zeros(NB, BS, HKV, D, dtype=torch.float8_e4m3fn, device=dev)
+        v8 = torch.zeros_like(k8)
+        ks = torch.ones(NB, BS, dtype=torch.float32, device=dev)
+        vs = torch.ones_like(ks)
+        ms16, _ = time_steps(torch, lambda: pa.store_kv_cache(k, v, kc, vc, slots), steps, warmup)
+        ms8, _ = time_steps(torch, lambda: pa.store_kv_cache(k, v, k8, v8, slots, ks, vs, "fp8"), steps, warmup)
+        out["tokens_%d" % n] = {"fp16_us": round(ms16 * 1e3, 2), "fp8_us": round(ms8 * 1e3, 2)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -284,6 +306,7 @@ def main():
         },
     }
     line["prefill_mfma"] = prefill
+    line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
