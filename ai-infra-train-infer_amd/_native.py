@@ -48,6 +48,7 @@ SIGNATURES = {
     "pa_set_decode_waves": (_int, [_int]),
     "pa_get_decode_waves": (_int, []),
     "pa_set_decode_pair_heads": (_int, [_int]),
+    "pa_set_prefill_waves": (_int, [_int]),
 }
 
 _lock = threading.Lock()

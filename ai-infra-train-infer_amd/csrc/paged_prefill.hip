@@ -34,6 +34,7 @@
 #include <stdio.h>
 
 #include <type_traits>
+#include <utility>
 
 namespace pa {
 
@@ -82,6 +83,45 @@ constexpr int kBN = 64;  // keys per tile
 // the same chunk index of 16 rows (MFMA A-operand reads of K) hit distinct banks, and (b) 4
 // consecutive rows differ in bits 2..3: the 4-row x 64-byte patch that 32 lanes fetch in one
 // pass of a transpose read of V spreads over 16 distinct chunk positions.
+// The same transpose read issued as opaque asm, for the tile loop of the fp16 path: the
+// compiler's wait-count pass cannot tell that the transpose-read builtin does not touch the buffer
+// that global_load_lds is filling, and drains every outstanding global load in front of it, in the
+// middle of the tile's arithmetic.  The result of an untracked read is not known to that pass
+// either: the caller waits with lds_wait<N> before use.  LDS operations complete in order, so the
+// extra outstanding reads only make the compiler's own lgkmcnt waits more conservative.
+template <int OFF>
+__device__ __forceinline__ half4_t tr_read_untracked(uint32_t lds_byte_addr) {
+  half4_t r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ half8_t b128_read_untracked(uint32_t lds_byte_addr) {
+  half8_t r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "n"(OFF));
+  return r;
+}
+// Waits until at most N LDS operations are outstanding; the operands are tied so that no consumer
+// of them can be scheduled above the wait.
+template <int N>
+__device__ __forceinline__ void lds_wait(half4_t& a, half4_t& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(half8_t& a, half8_t& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 template <int CPR>
 __device__ __forceinline__ constexpr int swz(int row) {
   return (((row & 3) << 2) | ((row >> 2) & 3)) & (CPR - 1);
@@ -133,15 +173,16 @@ constexpr int src_bytes() { return SRC == SRC_FP8 ? 1 : (SRC == SRC_F32 ? 4 : 2)
 
 // DIRECT: fp16 sources go global -> LDS with global_load_lds_dwordx4 (no staging registers, two
 // workgroups per CU); other source types are converted in registers on the way (one per CU).
-template <int D, int HPWG, int SRC>
-__global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_kernel(const PrefillParams p) {
+template <int D, int HPWG, int SRC, int W>
+__global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void paged_prefill_kernel(const PrefillParams p) {
+  constexpr int NT = 64 * W;              // threads per workgroup
   using L = PrefillLds<D>;
   constexpr bool DIRECT = SRC == SRC_F16;
   constexpr int KSTEPS = D / 16;          // MFMA k-steps over head_dim
   constexpr int MT = D / 32;              // 32-row tiles of O^T
-  constexpr int BM = 128 / HPWG;          // query tokens per workgroup
+  constexpr int BM = 32 * W / HPWG;       // query tokens per workgroup
   constexpr int CPR = D / 8;              // 8-element chunks per row
-  constexpr int NCH = kBN * CPR / 256;    // chunks per thread per tile (K and V each)
+  constexpr int NCH = kBN * CPR / NT;     // chunks per thread per tile (K and V each)
   constexpr int ES = src_bytes<SRC>();
   constexpr float NEG_INF = -INFINITY;
 
@@ -165,8 +206,8 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   if (tok0 >= lq) return;
   const int shift = lk - lq;  // row i sees keys <= i + shift
 
-  const int hslot = (HPWG == 2) ? (wave >> 1) : 0;
-  const int tsub = (HPWG == 2) ? (wave & 1) : wave;
+  const int hslot = (HPWG == 2) ? wave / (W / 2) : 0;
+  const int tsub = (HPWG == 2) ? wave % (W / 2) : wave;
   const int qhead = blockIdx.x * HPWG + hslot;
   const int kvh = (blockIdx.x * HPWG) / (p.num_q_heads / p.num_kv_heads);
   const int tokw0 = tok0 + tsub * 32;            // first token of this wave
@@ -210,7 +251,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   const int bt_last = max((int)p.bt_stride - 1, 0);
 
   // ---- staging: global -> (registers ->) LDS ---------------------------------------------------------
-  // chunk = 16 bytes of fp16 = 8 head-dim elements; thread `tid` moves chunks tid, tid+256, ...
+  // chunk = 16 bytes of fp16 = 8 head-dim elements; thread `tid` moves chunks tid, tid+NT, ...
   // i.e. one instruction of a wave covers 64 / CPR whole rows, contiguous in LDS.
   auto row_slot = [&](int key) -> int64_t {   // physical row of a key (clamped: never faults)
     const int kk = min(key, lk - 1);
@@ -230,14 +271,14 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   uint32_t lane_part[NCH];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    const int chunk = tid + 256 * c;
+    const int chunk = tid + NT * c;
     const int row = chunk / CPR;
     const int col = (chunk % CPR) ^ swz<CPR>(row);
     lane_part[c] = (uint32_t)(((lane / CPR) * token_elems + (int64_t)kvh * D + col * 8) * ES);
   }
   auto move_chunk = [&](int c, int buf, const uint8_t* kp, const uint8_t* vp, int64_t slot) {
     if constexpr (DIRECT) {
-      const int wbase = (256 * c + (tid & ~63)) * 8;   // LDS destination = wave base + lane * 16 bytes
+      const int wbase = (NT * c + (tid & ~63)) * 8;   // LDS destination = wave base + lane * 16 bytes
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
                                        (__attribute__((address_space(3))) void*)&lds.k[buf][wbase], 16, 0, 0);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
@@ -256,14 +297,14 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
   // load ever waits on another: lane l holds the entry of chunk group l % NCH of this wave.
   auto load_ids = [&](int t) -> int {
     if (!bt_row) return 0;
-    const int row0 = (256 * (lane % NCH) + 64 * wave) / CPR;
+    const int row0 = (NT * (lane % NCH) + 64 * wave) / CPR;
     return bt_row[min((t * kBN + row0) >> p.bs_log2, bt_last)];
   };
   auto fetch = [&](int t, int buf, int ids) {
     if (uniform_rows && (t + 1) * kBN <= lk) {
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
-        const int row0 = (256 * c + 64 * wave) / CPR;      // first row of this wave's instruction
+        const int row0 = (NT * c + 64 * wave) / CPR;      // first row of this wave's instruction
         const int key0 = t * kBN + row0;
         int64_t slot0;
         if (bt_row) {
@@ -279,7 +320,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-      const int chunk = tid + 256 * c;
+      const int chunk = tid + NT * c;
       const int row = chunk / CPR;
       const int col = (chunk % CPR) ^ swz<CPR>(row);   // head-dim chunk that belongs at this LDS position
       const int64_t slot = row_slot(t * kBN + row);    // rows past the sequence end re-read its last row (masked later)
@@ -291,7 +332,7 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     if constexpr (!DIRECT) {
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
-        const int chunk = tid + 256 * c;
+        const int chunk = tid + NT * c;
         *(half8_t*)&lds.k[buf][chunk * 8] = stage_k[c];
         *(half8_t*)&lds.v[buf][chunk * 8] = stage_v[c];
       }
@@ -319,6 +360,17 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
       v_off[mt][r] = row * D + ((chunk ^ swz<CPR>(row)) << 3) + 4 * (tr_i & 1);
     }
 
+  const uint32_t k_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&lds.k[0][0];
+  uint32_t k_addr[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) k_addr[ks] = k_base + 2u * (uint32_t)k_off[ks];
+  const uint32_t v_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&lds.v[0][0];
+  uint32_t v_addr[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 2; ++r) v_addr[mt][r] = v_base + 2u * (uint32_t)v_off[mt][r];
+
   // `buf` is a compile-time constant (the tile loop is unrolled by two) so that every LDS read
   // below is "loop-invariant register + immediate offset".
   auto compute = [&](int t, auto buf_tag) {
@@ -327,14 +379,38 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     // ---- S^T = K . Q^T : two 32-key tiles -------------------------------------------------------
     float16_t s[2];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+    if constexpr (DIRECT) {
+      // All K fragments of the first 32-key half are requested at once and those of the second
+      // half as the first are consumed, so a product never waits for a read issued just before it.
+      constexpr int OFF0 = buf * kBN * D * 2, OFF1 = OFF0 + 32 * D * 2;
+      half8_t ka[KSTEPS], kb[KSTEPS];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * D + k_off[ks]];
-        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], s[kt], 0, 0, 0);
-      }
+      for (int ks = 0; ks < KSTEPS; ++ks) ka[ks] = b128_read_untracked<OFF0>(k_addr[ks]);
+      static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int ks = 2 * decltype(j_tag)::value;
+        lds_wait<KSTEPS - 2>(ka[ks], ka[ks + 1]);   // outstanding: the rest of ka and what is issued of kb
+        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks], qreg[ks], s[0], 0, 0, 0);
+        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks + 1], qreg[ks + 1], s[0], 0, 0, 0);
+        kb[ks] = b128_read_untracked<OFF1>(k_addr[ks]);
+        kb[ks + 1] = b128_read_untracked<OFF1>(k_addr[ks + 1]);
+      });
+      static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
+        constexpr int ks = 2 * decltype(j_tag)::value;
+        lds_wait<KSTEPS - 2 - ks>(kb[ks], kb[ks + 1]);
+        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks], qreg[ks], s[1], 0, 0, 0);
+        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks + 1], qreg[ks + 1], s[1], 0, 0, 0);
+      });
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * D + k_off[ks]];
+          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], s[kt], 0, 0, 0);
+        }
     }
     // ---- mask: only tiles that reach past the diagonal of this wave or the sequence end ---------
     const int wave_first_lim = tokw0 + shift;  // smallest row limit in the wave
@@ -385,16 +461,56 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
       }
     l_run += psum;
     // ---- O^T += V^T . P^T : four 16-key steps x MT row tiles ----------------------------------------
+    if constexpr (DIRECT) {
+      // untracked reads, one 16-key step ahead of the products that use them
+      half4_t lo[2][MT], hi[2][MT];
+      auto issue = [&](auto k2_tag) __attribute__((always_inline)) {
+        constexpr int k2 = decltype(k2_tag)::value;
+        constexpr int OFF = (buf * kBN * D + k2 * 16 * D) * 2;
 #pragma unroll
-    for (int k2 = 0; k2 < 4; ++k2) {
+        for (int mt = 0; mt < MT; ++mt) {
+          lo[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][0]);
+          hi[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][1]);
+        }
+      };
+      auto multiply = [&](auto k2_tag) __attribute__((always_inline)) {
+        constexpr int k2 = decltype(k2_tag)::value;
+        // reads return in order: this step's have all landed once no more than the next step's
+        // 2 MT are outstanding.  volatile asm statements keep their order, so tying the other
+        // registers to empty statements after the wait holds their consumers below it too.
+        if constexpr (k2 < 3) lds_wait<2 * MT>(lo[k2 & 1][0], hi[k2 & 1][0]);
+        else lds_wait<0>(lo[k2 & 1][0], hi[k2 & 1][0]);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const half4_t lo = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][0]]);
-        const half4_t hi = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][1]]);
-        half8_t a;
-        a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
-        a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
+        for (int mt = 1; mt < MT; ++mt) asm volatile("" : "+v"(lo[k2 & 1][mt]), "+v"(hi[k2 & 1][mt]));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const half4_t l4 = lo[k2 & 1][mt], h4 = hi[k2 & 1][mt];
+          half8_t a;
+          a[0] = l4[0]; a[1] = l4[1]; a[2] = l4[2]; a[3] = l4[3];
+          a[4] = h4[0]; a[5] = h4[1]; a[6] = h4[2]; a[7] = h4[3];
+          o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
+        }
+      };
+      issue(std::integral_constant<int, 0>{});
+      issue(std::integral_constant<int, 1>{});
+      multiply(std::integral_constant<int, 0>{});
+      issue(std::integral_constant<int, 2>{});
+      multiply(std::integral_constant<int, 1>{});
+      issue(std::integral_constant<int, 3>{});
+      multiply(std::integral_constant<int, 2>{});
+      multiply(std::integral_constant<int, 3>{});
+    } else {
+#pragma unroll
+      for (int k2 = 0; k2 < 4; ++k2) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const half4_t lo = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][0]]);
+          const half4_t hi = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][1]]);
+          half8_t a;
+          a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
+          a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
+          o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
+        }
       }
     }
   };
@@ -451,9 +567,9 @@ __global__ __launch_bounds__(256, (SRC == SRC_F16 ? 2 : 1)) void paged_prefill_k
     }
 }
 
-template <int D, int HPWG, int SRC>
+template <int D, int HPWG, int SRC, int W>
 static int launch_prefill(const PrefillParams& p, dim3 grid, hipStream_t st) {
-  auto kern = paged_prefill_kernel<D, HPWG, SRC>;
+  auto kern = paged_prefill_kernel<D, HPWG, SRC, W>;
   const size_t smem = sizeof(PrefillLds<D>);
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
@@ -461,23 +577,37 @@ static int launch_prefill(const PrefillParams& p, dim3 grid, hipStream_t st) {
       return fail(PA_ERR_LAUNCH, "pa_prefill: cannot raise the dynamic LDS limit");
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, p);
+  hipLaunchKernelGGL(kern, grid, dim3(64 * W), smem, st, p);
   return PA_OK;
 }
 
-template <int D, int HPWG>
+template <int D, int HPWG, int W>
 static int launch_prefill_src(const PrefillParams& p, dim3 grid, int src, hipStream_t st) {
   switch (src) {
-    case SRC_F16: return launch_prefill<D, HPWG, SRC_F16>(p, grid, st);
-    case SRC_BF16: return launch_prefill<D, HPWG, SRC_BF16>(p, grid, st);
-    case SRC_FP8: return launch_prefill<D, HPWG, SRC_FP8>(p, grid, st);
-    default: return launch_prefill<D, HPWG, SRC_F32>(p, grid, st);
+    case SRC_F16: return launch_prefill<D, HPWG, SRC_F16, W>(p, grid, st);
+    case SRC_BF16: return launch_prefill<D, HPWG, SRC_BF16, W>(p, grid, st);
+    case SRC_FP8: return launch_prefill<D, HPWG, SRC_FP8, W>(p, grid, st);
+    default: return launch_prefill<D, HPWG, SRC_F32, W>(p, grid, st);
   }
 }
+
+template <int D, int W>
+static int launch_prefill_hpwg(const PrefillParams& p, dim3 grid, int hpwg, int src, hipStream_t st) {
+  return hpwg == 2 ? launch_prefill_src<D, 2, W>(p, grid, src, st) : launch_prefill_src<D, 1, W>(p, grid, src, st);
+}
+
+static int g_prefill_waves = 0;  // 0 = chosen per launch
 
 }  // namespace pa
 
 using namespace pa;
+
+extern "C" int pa_set_prefill_waves(int waves) {
+  if (waves != 0 && waves != 4 && waves != 8)
+    return fail(PA_ERR_BAD_ARG, "pa_set_prefill_waves: waves per workgroup must be 0 (automatic), 4 or 8");
+  g_prefill_waves = waves;
+  return PA_OK;
+}
 
 extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                           const void* v_cache, const float* k_scale, const float* v_scale,
@@ -533,7 +663,15 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
 
   const int g = (int)(num_q_heads / num_kv_heads);
   const int hpwg = (g % 2 == 0) ? 2 : 1;
-  const int bm = 128 / hpwg;
+  // 8 waves per workgroup share each K/V tile between twice as many query rows, which halves
+  // the bytes every CU pulls through its L1; worth it once such workgroups fill most of the chip.
+  int w = g_prefill_waves;
+  if (w == 0) {
+    const int64_t bm8 = 256 / hpwg;
+    const int64_t wgs8 = (num_q_heads / hpwg) * ((max_seqlen_q + bm8 - 1) / bm8) * num_seqs;
+    w = (max_seqlen_q > bm8 / 2 && wgs8 >= 192) ? 8 : 4;
+  }
+  const int bm = 32 * w / hpwg;            // query tokens per workgroup
 
   PrefillParams p;
   p.q = q;
@@ -560,9 +698,9 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (head_dim == 128)
-    rc = hpwg == 2 ? launch_prefill_src<128, 2>(p, grid, src, st) : launch_prefill_src<128, 1>(p, grid, src, st);
+    rc = w == 8 ? launch_prefill_hpwg<128, 8>(p, grid, hpwg, src, st) : launch_prefill_hpwg<128, 4>(p, grid, hpwg, src, st);
   else
-    rc = hpwg == 2 ? launch_prefill_src<64, 2>(p, grid, src, st) : launch_prefill_src<64, 1>(p, grid, src, st);
+    rc = w == 8 ? launch_prefill_hpwg<64, 8>(p, grid, hpwg, src, st) : launch_prefill_hpwg<64, 4>(p, grid, hpwg, src, st);
   if (rc != PA_OK) return rc;
   return check_launch("pa_prefill");
 }

@@ -207,6 +207,9 @@ int pa_get_decode_waves(void);
 /* Tunable: let one wavefront serve two adjacent KV heads when a head's row is <= 128 bytes
  * (fp8 at head_dim 128, any dtype at head_dim 64).  On by default. */
 int pa_set_decode_pair_heads(int enable);
+/* Tunable of the prefill launch: waves per workgroup, 4 (64 query tokens x 2 heads per K/V tile)
+ * or 8 (128 x 2), or 0 = chosen per launch from the grid size (default). Returns PA_OK or BAD_ARG. */
+int pa_set_prefill_waves(int waves_per_workgroup);
 
 #ifdef __cplusplus
 }

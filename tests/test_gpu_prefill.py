@@ -56,6 +56,14 @@ def check(got, want, kind="fp16"):
     torch.testing.assert_close(got.float(), want.float(), rtol=rtol, atol=atol)
 
 
+@pytest.fixture(params=[4, 8])
+def waves(request, lib):
+    """Force the 4-wave or the 8-wave workgroup shape of the prefill kernel; automatic afterwards."""
+    assert lib.pa_set_prefill_waves(request.param) == 0
+    yield request.param
+    assert lib.pa_set_prefill_waves(0) == 0
+
+
 def test_config5a_chunked_prefill_bf16_q_fp16_kv(pa, gpu):
     c = make_prefill(1005, [2048] * 8, [512] * 8, 8 * 160 + 32, q_dtype=torch.bfloat16)
     got = gpu_prefill(pa, c, gpu)
@@ -64,7 +72,7 @@ def test_config5a_chunked_prefill_bf16_q_fp16_kv(pa, gpu):
 
 
 @pytest.mark.parametrize("cache", ["fp16", "fp8", "bf16"])
-def test_ragged_chunks(pa, gpu, cache):
+def test_ragged_chunks(pa, gpu, cache, waves):
     cached = [0, 5, 64, 100, 0, 333, 17]
     new = [1, 63, 64, 65, 200, 7, 130]
     c = make_prefill(60, cached, new, 96, cache=cache)
@@ -72,13 +80,13 @@ def test_ragged_chunks(pa, gpu, cache):
 
 
 @pytest.mark.parametrize("hq,hkv,d", [(16, 8, 128), (8, 8, 128), (16, 4, 128), (8, 2, 64), (4, 4, 64)])
-def test_head_shapes(pa, gpu, hq, hkv, d):
+def test_head_shapes(pa, gpu, hq, hkv, d, waves):
     c = make_prefill(61 + hq + d, [40, 0, 129], [70, 150, 3], 48, num_heads=hq, num_kv_heads=hkv, head_dim=d)
     check(gpu_prefill(pa, c, gpu), oracle_prefill(c, upcast=True))
 
 
 @pytest.mark.parametrize("bs", [8, 32])
-def test_block_sizes(pa, gpu, bs):
+def test_block_sizes(pa, gpu, bs, waves):
     c = make_prefill(62, [bs * 3 + 1, 0], [100, 77], 64, block_size=bs)
     check(gpu_prefill(pa, c, gpu), oracle_prefill(c, upcast=True))
 
@@ -155,6 +163,12 @@ def test_module_forward_prefill_then_decode(pa, gpu):
     torch.cuda.synchronize()
     check(out.cpu(), want)
     assert torch.equal(d["k_cache"].cpu().view(torch.int16), c["k_cache"].view(torch.int16))
+
+
+def test_waves_tunable_rejects_other_values(lib, gpu):
+    assert lib.pa_set_prefill_waves(6) != 0
+    assert b"pa_set_prefill_waves" in lib.pa_last_error()
+    assert lib.pa_set_prefill_waves(0) == 0
 
 
 def test_c_abi_argument_errors(lib, gpu):
