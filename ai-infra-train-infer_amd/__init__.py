@@ -9,7 +9,8 @@ The directory name contains a hyphen, so import it through the `ai_infra_train_i
 loader module at the repository root.
 """
 from .context import InferenceContext, set_context, get_context, reset_context
-from .kv_cache import BlockPool, HAS_FP8, _FP8_DTYPE
+from .kv_cache import Block, BlockPool, BlockTable, KVCacheManager, HAS_FP8, _FP8_DTYPE
+from .prefix_cache import PrefixCache, CachedBlock
 from .attention import (
     PagedAttention,
     PartitionedPagedAttention,
@@ -26,7 +27,7 @@ from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "BlockPool", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",

@@ -201,6 +201,20 @@ int pa_fp8_e4m3_to_f32(const void* src, float* dst, int64_t n, void* stream);
  */
 int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
 
+/*
+ * Copy whole cache blocks inside one pool tensor laid out [num_planes][num_blocks][block_bytes]
+ * (planes plane_stride_bytes apart): for every plane and every pair i, block pairs[2i+1] := block
+ * pairs[2i].  The K/V tensor of a BlockPool is one such tensor with 2 x layers planes, each fp8
+ * scale tensor one with `layers` planes.  pairs is a device int32 array; pairs with an id outside
+ * [0, num_blocks) or src == dst are skipped; no destination may be another pair's source.
+ * Replaces: nothing the reference ships.  Its blocks carry a ref_count for prefix sharing
+ * (src/inference/kv_cache.py:42-62, 195-212) but are never shared, and its K-sample path notes
+ * that skipping the shared prompt needs block sharing / copying first
+ * (src/inference/engine.py:1108-1113); this is the copy half of copy-on-write.
+ */
+int pa_copy_blocks(void* pool, int64_t num_planes, int64_t plane_stride_bytes, int64_t block_bytes,
+                   int64_t num_blocks, const int32_t* pairs, int64_t num_pairs, void* stream);
+
 /* Tunables of the decode launch (waves per workgroup: 1, 2, 4 or 8). Returns PA_OK or BAD_ARG. */
 int pa_set_decode_waves(int waves_per_workgroup);
 int pa_get_decode_waves(void);
