@@ -150,6 +150,77 @@ def store_kv_cache(
 _WORKSPACES = {}
 
 
+def qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, positions,
+                       k_cache=None, v_cache=None, slot_mapping=None, k_scale=None, v_scale=None,
+                       cache_dtype="fp16", return_k=False):
+    """Per-head RMSNorm of q and k, rotary embedding of both, and the paged cache write of k and
+    v in one launch: what a Qwen3 attention block does between its projections and the
+    attention call (src/distributed/tensor_parallel.py:78-84, 394-419, 453-464) followed by
+    store_kv_cache (src/inference/attention.py:44-183).
+
+    q [T, Hq, D], k / v [T, Hkv, D] (views with a token stride are fine), weights [D],
+    inv_freq fp32 [D/2], positions int64 [T].  Returns (q_out, k_out) with k_out None unless
+    return_k.  Without caches (or without a slot_mapping) nothing is written to the pool.
+    """
+    _require_gpu(q, "qk_norm_rope_store")
+    lib = _native.load()
+    if q.dim() != 3 or k.dim() != 3 or q.shape[0] != k.shape[0] or q.shape[2] != k.shape[2]:
+        raise RuntimeError("qk_norm_rope_store: expected q [T,Hq,D] and k [T,Hkv,D], got %s and %s"
+                           % (tuple(q.shape), tuple(k.shape)))
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if k.dtype != q.dtype or (v is not None and v.dtype != q.dtype):
+        raise RuntimeError("qk_norm_rope_store: q, k and v dtypes differ")
+    q, qs = _rows(q, "qk_norm_rope_store")
+    k, ks_ = _rows(k, "qk_norm_rope_store")
+    if q_norm_weight.numel() != d or k_norm_weight.numel() != d or q_norm_weight.dtype != k_norm_weight.dtype:
+        raise RuntimeError("qk_norm_rope_store: norm weights must both be [head_dim] of one dtype")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != d // 2:
+        raise RuntimeError("qk_norm_rope_store: inv_freq must be fp32 [head_dim / 2]")
+    if positions.numel() != n:
+        raise RuntimeError("qk_norm_rope_store: positions has %d entries for %d tokens" % (positions.numel(), n))
+    positions = positions.to(torch.int64).contiguous()
+    q_out = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
+    k_out = torch.empty((n, hkv, d), dtype=q.dtype, device=q.device) if return_k else None
+    write = k_cache is not None and slot_mapping is not None
+    vs_ = 0
+    kv_code = _code(q.dtype, "qk_norm_rope_store")
+    total_slots = 0
+    if write:
+        _check_cache(k_cache, v_cache, "qk_norm_rope_store")
+        if tuple(k_cache.shape[2:]) != (hkv, d) or v is None or v.shape != k.shape:
+            raise RuntimeError("qk_norm_rope_store: k/v %s do not match the cache %s"
+                               % (tuple(k.shape), tuple(k_cache.shape)))
+        v, vs_ = _rows(v, "qk_norm_rope_store")
+        total_slots = k_cache.shape[0] * k_cache.shape[1]
+        if slot_mapping.numel() != n:
+            raise RuntimeError("qk_norm_rope_store: slot_mapping has %d entries for %d tokens"
+                               % (slot_mapping.numel(), n))
+        slot_mapping = _int32(slot_mapping, "qk_norm_rope_store")
+        if cache_dtype == "fp8" and HAS_FP8:
+            if k_cache.dtype != _FP8_DTYPE or k_scale is None or v_scale is None:
+                raise RuntimeError("qk_norm_rope_store: cache_dtype='fp8' needs float8_e4m3fn caches and scales")
+            kv_code = _native.DTYPE_FP8_E4M3
+        elif k_cache.dtype != q.dtype:
+            raise RuntimeError("qk_norm_rope_store: cache dtype %s differs from the activations' %s"
+                               % (k_cache.dtype, q.dtype))
+    if n == 0:
+        return q_out, k_out
+    fp8 = kv_code == _native.DTYPE_FP8_E4M3
+    rc = lib.pa_qk_norm_rope_store(
+        q.data_ptr(), k.data_ptr(), v.data_ptr() if write else None, _code(q.dtype, "qk_norm_rope_store"),
+        qs, ks_, vs_, q_norm_weight.data_ptr(), k_norm_weight.data_ptr(),
+        _code(q_norm_weight.dtype, "qk_norm_rope_store"), float(eps), inv_freq.data_ptr(), positions.data_ptr(),
+        q_out.data_ptr(), hq * d, k_out.data_ptr() if return_k else None, hkv * d,
+        k_cache.data_ptr() if write else None, v_cache.data_ptr() if write else None,
+        k_scale.data_ptr() if (write and fp8) else None, v_scale.data_ptr() if (write and fp8) else None,
+        kv_code, slot_mapping.data_ptr() if write else None, n, hq, hkv, d, total_slots, _stream_ptr(q.device))
+    if rc != 0:
+        raise RuntimeError("pa_qk_norm_rope_store failed (%d): %s"
+                           % (rc, lib.pa_last_error().decode("utf-8", "replace")))
+    return q_out, k_out
+
+
 def _workspace(device, nbytes):
     """Per (device, stream) scratch for the partition partials; grows, never shrinks."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
@@ -342,6 +413,21 @@ class PagedAttention(nn.Module):
                            cache_dtype=self.cache_dtype)
         if ctx.is_prefill:
             return self._prefill_attention(q, k, v, ctx)
+        return self._decode_attention(q, ctx)
+
+    def forward_fused(self, q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, positions):
+        """forward() for projections that still need their per-head RMSNorm and rotary embedding:
+        norm, rotation and the cache write run as one kernel, then attention as in forward()."""
+        ctx = get_context()
+        write = self.k_cache is not None and ctx.slot_mapping is not None
+        dense_k = ctx.is_prefill and not (ctx.block_tables is not None and self.k_cache is not None)
+        q, k_rot = qk_norm_rope_store(
+            q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, positions,
+            k_cache=self.k_cache if write else None, v_cache=self.v_cache if write else None,
+            slot_mapping=ctx.slot_mapping if write else None, k_scale=self.k_scale, v_scale=self.v_scale,
+            cache_dtype=self.cache_dtype, return_k=dense_k)
+        if ctx.is_prefill:
+            return self._prefill_attention(q, k_rot, v, ctx)
         return self._decode_attention(q, ctx)
 
     def _scales(self):

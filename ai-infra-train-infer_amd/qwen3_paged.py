@@ -6,8 +6,9 @@ the module a model runner binds caches to (model_runner.py:102-116) and calls as
 `model(input_ids, positions=positions)` (model_runner.py:162).  Block structure follows the
 reference's Qwen3 definition (src/distributed/tensor_parallel.py:307-543): RMSNorm -> q/k/v
 projections -> per-head q/k RMSNorm -> RoPE (half rotation, theta 1e6) -> attention -> o_proj,
-then RMSNorm -> SwiGLU MLP.  GEMMs and norms are plain torch-ROCm ops; only the attention and
-the KV write go through the HIP kernels.  Nothing in forward() synchronises with the host, so a
+then RMSNorm -> SwiGLU MLP.  GEMMs and the layer norms are plain torch-ROCm ops; the per-head
+q/k norm, the rotation and the KV write are one HIP kernel (`fused_qk`, on by default; off =
+the same steps as separate torch ops), attention another.  Nothing in forward() synchronises with the host, so a
 decode step can be captured in a HIP graph.
 """
 from dataclasses import dataclass
@@ -34,6 +35,7 @@ class Qwen3PagedConfig:
     rms_norm_eps: float = 1e-6
     cache_dtype: str = "fp16"
     partition_size: int = 0        # > 0: use PartitionedPagedAttention with this size
+    fused_qk: bool = True          # q/k norm + RoPE + cache write as one kernel
 
 
 class RMSNorm(nn.Module):
@@ -74,7 +76,7 @@ class Qwen3PagedLayer(nn.Module):
         self.gate_up_proj = nn.Linear(cfg.hidden_size, 2 * cfg.intermediate_size, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
 
-    def forward(self, x, cos, sin):
+    def forward(self, x, cos, sin, positions=None, inv_freq=None):
         cfg = self.cfg
         t = x.shape[0]
         q_dim, kv_dim = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
@@ -82,9 +84,13 @@ class Qwen3PagedLayer(nn.Module):
         q = qkv[:, :q_dim].view(t, cfg.num_heads, cfg.head_dim)
         k = qkv[:, q_dim:q_dim + kv_dim].view(t, cfg.num_kv_heads, cfg.head_dim)
         v = qkv[:, q_dim + kv_dim:].view(t, cfg.num_kv_heads, cfg.head_dim)
-        q = apply_rope(self.q_norm(q), cos, sin)
-        k = apply_rope(self.k_norm(k), cos, sin)
-        a = self.attn(q, k, v)                      # writes k, v into the paged cache, then attends
+        if cfg.fused_qk and positions is not None and x.is_cuda:
+            a = self.attn.forward_fused(q, k, v, self.q_norm.weight, self.k_norm.weight,
+                                        cfg.rms_norm_eps, inv_freq, positions)
+        else:
+            q = apply_rope(self.q_norm(q), cos, sin)
+            k = apply_rope(self.k_norm(k), cos, sin)
+            a = self.attn(q, k, v)                  # writes k, v into the paged cache, then attends
         x = x + self.o_proj(a.reshape(t, q_dim))
         gu = self.gate_up_proj(self.post_attention_layernorm(x))
         gate, up = gu[:, :cfg.intermediate_size], gu[:, cfg.intermediate_size:]
@@ -114,10 +120,13 @@ class Qwen3PagedModel(nn.Module):
     def forward(self, input_ids, positions=None):
         if positions is None:
             positions = torch.arange(input_ids.shape[0], device=input_ids.device)
-        cos, sin = self.rope_tables(positions)
+        fused = self.cfg.fused_qk and input_ids.is_cuda
+        cos, sin = (None, None) if fused else self.rope_tables(positions)
         x = self.embed_tokens(input_ids)
+        # a model cast with .half() carries its frequency table in 16 bits; both paths use those values
+        inv_freq = self.inv_freq.float()
         for layer in self.layers:
-            x = layer(x, cos, sin)
+            x = layer(x, cos, sin, positions, inv_freq)
         ctx = get_context()
         if ctx.is_prefill and ctx.cu_seqlens_q is not None:
             x = x[(ctx.cu_seqlens_q[1:] - 1).long()]

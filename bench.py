@@ -169,6 +169,54 @@ def kv_store_times(pa, torch, dev, steps, warmup):
     return out
 
 
+def fused_qk_times(pa, torch, dev, steps, warmup):
+    """Per-head q/k RMSNorm + rotary embedding + paged cache write of one layer: the fused kernel
+    beside the same steps as separate torch ops followed by store_kv_cache, for one decode step
+    (64 tokens) and one prefill chunk (4096 tokens), FP16 cache.  Microseconds; for 4096 tokens also
+    the achieved bandwidth over the algorithmic bytes (q, k, v read once; q, and k, v to the cache,
+    written once)."""
+    from ai_infra_train_infer_amd.qwen3_paged import RMSNorm, apply_rope
+    HQ, HKV, D, BS, NB = 16, 8, 128, 16, 4096 // 16 + 64
+    g = torch.Generator(device=dev).manual_seed(8)
+    qn, kn = RMSNorm(D, 1e-6).to(dev).half(), RMSNorm(D, 1e-6).to(dev).half()
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))).to(dev)
+    out = {}
+    for n in (64, 4096):
+        qkv = torch.randn(n, (HQ + 2 * HKV) * D, generator=g, device=dev, dtype=torch.float32).half()
+        q = qkv[:, :HQ * D].view(n, HQ, D)
+        k = qkv[:, HQ * D:(HQ + HKV) * D].view(n, HKV, D)
+        v = qkv[:, (HQ + HKV) * D:].view(n, HKV, D)
+        pos = torch.randint(0, 4096, (n,), generator=g, device=dev)
+        slots = torch.randperm(NB * BS, generator=g, device=dev)[:n].to(torch.int32)
+        kc = torch.zeros(NB, BS, HKV, D, dtype=torch.float16, device=dev)
+        vc = torch.zeros_like(kc)
+
+        def fused():
+            pa.qk_norm_rope_store(q, k, v, qn.weight, kn.weight, 1e-6, inv_freq, pos, k_cache=kc, v_cache=vc,
+                                  slot_mapping=slots)
+
+        def separate():
+            freqs = pos.float()[:, None] * inv_freq[None, :]
+            emb = torch.cat([freqs, freqs], dim=-1)
+            cos, sin = emb.cos()[:, None, :], emb.sin()[:, None, :]
+            q2 = apply_rope(qn(q), cos, sin)
+            k2 = apply_rope(kn(k), cos, sin)
+            pa.store_kv_cache(k2, v, kc, vc, slots)
+            return q2
+
+        with torch.inference_mode():
+            ms_f, _ = time_steps(torch, fused, steps, warmup)
+            ms_s, _ = time_steps(torch, separate, steps, warmup)
+        rec = {"fused_us": round(ms_f * 1e3, 2), "separate_ops_us": round(ms_s * 1e3, 2),
+               "speedup": round(ms_s / ms_f, 1)}
+        if n == 4096:
+            alg = n * (HQ + 2 * HKV) * D * 2 * 2
+            rec["algorithmic_bytes"] = alg
+            rec["gbps"] = round(alg / ms_f / 1e6, 1)
+        out["tokens_%d" % n] = rec
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -307,6 +355,7 @@ def main():
     }
     line["prefill_mfma"] = prefill
     line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
+    line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))

@@ -202,6 +202,32 @@ int pa_fp8_e4m3_to_f32(const void* src, float* dst, int64_t n, void* stream);
 int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
 
 /*
+ * Per-head RMSNorm of q and k, rotary embedding of both, and the paged cache write of k and v,
+ * for num_tokens tokens in one launch.
+ *   q [T, Hq, D], k, v [T, Hkv, D] in `dtype` (f16 / bf16 / f32), token strides in elements
+ *   y = w * (x * rsqrt(mean(x^2) + eps)) per head row in fp32, rounded to `dtype`;
+ *   then [y1, y2] -> [y1 cos - y2 sin, y2 cos + y1 sin] on the two halves of the row, with
+ *   angle = float(positions[t]) * inv_freq[i], in fp32, rounded to `dtype`
+ *   q_out [T, Hq, D] receives q; k_out (optional, may be NULL) a dense copy of k
+ *   k_cache / v_cache [total_slots, Hkv, D]: slot_mapping[t] receives rotated k and raw v, as
+ *   pa_kv_store (kv_dtype == dtype) or pa_kv_store_fp8 (kv_dtype == PA_DTYPE_FP8_E4M3, per-token
+ *   scales to k_scale / v_scale) would write them; slot < 0 or >= total_slots: no cache write.
+ *   k_cache == NULL: no cache write at all (v, v_cache, scales, slot_mapping unused).
+ * head_dim 64 or 128; Hkv * D * sizeof(dtype) <= 8192.
+ * Replaces: RMSNorm.forward on q and k (src/distributed/tensor_parallel.py:78-84, used at
+ * :453-454), _apply_rotary_emb (:394-419, used at :457-464) and store_kv_cache
+ * (src/inference/attention.py:44-183) of one attention layer.
+ */
+int pa_qk_norm_rope_store(const void* q, const void* k, const void* v, int dtype, int64_t q_token_stride,
+                          int64_t k_token_stride, int64_t v_token_stride, const void* q_norm_weight,
+                          const void* k_norm_weight, int weight_dtype, float eps, const float* inv_freq,
+                          const int64_t* positions, void* q_out, int64_t q_out_token_stride, void* k_out,
+                          int64_t k_out_token_stride, void* k_cache, void* v_cache, float* k_scale,
+                          float* v_scale, int kv_dtype, const int32_t* slot_mapping, int64_t num_tokens,
+                          int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t total_slots,
+                          void* stream);
+
+/*
  * Copy whole cache blocks inside one pool tensor laid out [num_planes][num_blocks][block_bytes]
  * (planes plane_stride_bytes apart): for every plane and every pair i, block pairs[2i+1] := block
  * pairs[2i].  The K/V tensor of a BlockPool is one such tensor with 2 x layers planes, each fp8

@@ -41,11 +41,11 @@ def dense_reference_logits(model, token_ids):
     return model.lm_head(model.norm(x[-1:]))[0]
 
 
-def small_model(pa, cache_dtype="fp16", partition_size=0, seed=0):
+def small_model(pa, cache_dtype="fp16", partition_size=0, seed=0, fused_qk=True):
     torch.manual_seed(seed)
     cfg = pa.Qwen3PagedConfig(vocab_size=512, hidden_size=256, intermediate_size=512, num_layers=2,
                               num_heads=4, num_kv_heads=2, head_dim=64, cache_dtype=cache_dtype,
-                              partition_size=partition_size)
+                              partition_size=partition_size, fused_qk=fused_qk)
     return pa.Qwen3PagedModel(cfg).eval()
 
 
@@ -144,6 +144,28 @@ def test_chunked_prefill_over_cached_prefix(pa, gpu):
         close(final[i], dense_reference_logits(ref_model, s["token_ids"]))
 
 
+@pytest.mark.parametrize("cache_dtype", ["fp16", "fp8"])
+def test_fused_qk_norm_rope_store_equals_the_separate_ops(pa, gpu, cache_dtype):
+    fused = Session(pa, small_model(pa, cache_dtype, seed=6, fused_qk=True), gpu, cache_dtype=cache_dtype)
+    plain = Session(pa, small_model(pa, cache_dtype, seed=6, fused_qk=False), gpu, cache_dtype=cache_dtype)
+    g = torch.Generator().manual_seed(7)
+    for n in (21, 64, 50):
+        p = torch.randint(0, 512, (n,), generator=g).tolist()
+        fused.add(p)
+        plain.add(p)
+    tol = 4e-2 if cache_dtype == "fp8" else 1e-2
+    close(fused.prefill(chunk=32)[0], plain.prefill(chunk=32)[0].cpu(), tol)       # first chunk: no prefix, dense K
+    close(fused.prefill()[0], plain.prefill()[0].cpu(), tol)                       # rest: over the cached prefix
+    for step in range(3):
+        nxt = torch.randint(0, 512, (3,), generator=g).tolist()
+        close(fused.decode(nxt), plain.decode(nxt).cpu(), tol)
+    if cache_dtype == "fp16":
+        blk = fused.seqs[1]["block_table"][0]
+        assert blk == plain.seqs[1]["block_table"][0]
+        torch.testing.assert_close(fused.pool.kv_cache_tensor[:, 0, blk].float().cpu(),
+                                   plain.pool.kv_cache_tensor[:, 0, blk].float().cpu(), rtol=1e-3, atol=2e-3)
+
+
 def test_graph_replay_equals_eager_on_every_replay(pa, gpu):
     model = small_model(pa, seed=3)
     eager = Session(pa, model, gpu)
@@ -190,18 +212,23 @@ def test_config5b_qwen3_0p6b_shaped_decode_step(pa, gpu):
     seqs = [{"token_ids": [1] * CTX, "block_table": perm[b].tolist()} for b in range(B)]
     grabbed = {}
     check_layers = (0, 9, 27)
-    hooks = []
-    for l in check_layers:
-        def hook(mod, args, out, l=l):
-            grabbed[l] = (args[0].detach().clone(), out.detach().clone())
-        hooks.append(model.layers[l].attn.register_forward_hook(hook))
+    restore = []
+    for l in check_layers:               # record the query that reaches the attention kernel and its output
+        attn = model.layers[l].attn
+        inner = attn._decode_attention
+        def spy(q, ctx, l=l, inner=inner):
+            out = inner(q, ctx)
+            grabbed[l] = (q.detach().clone(), out.detach().clone())
+            return out
+        attn._decode_attention = spy
+        restore.append(attn)
     ids, pos = runner.prepare_decode(seqs)
     tables = pa.get_context().block_tables.cpu()
     lens = pa.get_context().context_lens.cpu()
     logits = runner.run(ids, pos, is_prefill=False)
     torch.cuda.synchronize()
-    for h in hooks:
-        h.remove()
+    for attn in restore:
+        del attn._decode_attention
     assert tuple(logits.shape) == (B, cfg.vocab_size) and torch.isfinite(logits).all()
     for l in check_layers:
         q, out = grabbed[l]
