@@ -16,6 +16,7 @@ from .attention import (
     PartitionedPagedAttention,
     store_kv_cache,
     qk_norm_rope_store,
+    sample_tokens,
     paged_decode,
     paged_prefill,
     choose_partition,
@@ -29,7 +30,7 @@ from . import _native
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
     "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "HAS_FP8",
-    "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store",
+    "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",
     "ModelRunner", "ModelRunnerConfig", "Qwen3PagedConfig", "Qwen3PagedModel",

@@ -48,6 +48,7 @@ SIGNATURES = {
     "pa_qk_norm_rope_store": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _int, _f32, _ptr,
                                      _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64,
                                      _i64, _i64, _i64, _i64, _ptr]),
+    "pa_sample": (_int, [_ptr, _int, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr]),
     "pa_copy_blocks": (_int, [_ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "pa_set_decode_waves": (_int, [_int]),
     "pa_get_decode_waves": (_int, []),

@@ -221,6 +221,35 @@ def qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, pos
     return q_out, k_out
 
 
+def sample_tokens(logits, temperature=0.7, top_p=0.9, uniforms=None, generator=None):
+    """One token id per row of logits [batch, vocab] -> int64 [batch] on the same device, without
+    a sort and without synchronising with the host (src/inference/model_runner.py:590-634).
+    temperature <= 0 is greedy.  uniforms: fp32 [batch] in [0, 1) for a reproducible draw; by
+    default drawn here from `generator` (or the device's default generator)."""
+    _require_gpu(logits, "sample_tokens")
+    if logits.dim() != 2:
+        raise RuntimeError("sample_tokens: expected [batch, vocab], got %s" % (tuple(logits.shape),))
+    lib = _native.load()
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    b, vocab = logits.shape
+    out = torch.empty(b, dtype=torch.int64, device=logits.device)
+    if b == 0:
+        return out
+    if temperature > 0:
+        if uniforms is None:
+            uniforms = torch.rand(b, device=logits.device, dtype=torch.float32, generator=generator)
+        if uniforms.numel() != b or uniforms.dtype != torch.float32 or not uniforms.is_cuda:
+            raise RuntimeError("sample_tokens: uniforms must be fp32 [batch] on the GPU")
+        uniforms = uniforms.contiguous()
+    rc = lib.pa_sample(logits.data_ptr(), _code(logits.dtype, "sample_tokens"), logits.stride(0) if b > 1 else vocab,
+                       b, vocab, float(temperature), float(top_p),
+                       uniforms.data_ptr() if temperature > 0 else None, out.data_ptr(), _stream_ptr(logits.device))
+    if rc != 0:
+        raise RuntimeError("pa_sample failed (%d): %s" % (rc, lib.pa_last_error().decode("utf-8", "replace")))
+    return out
+
+
 def _workspace(device, nbytes):
     """Per (device, stream) scratch for the partition partials; grows, never shrinks."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)

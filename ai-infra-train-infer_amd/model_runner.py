@@ -189,6 +189,16 @@ class ModelRunner:
         reset_context()
         return logits
 
+    # ---------------------------------------------------------------- sampling
+
+    def sample(self, logits: torch.Tensor, temperature: float = 0.7, top_p: float = 0.9,
+               uniforms: Optional[torch.Tensor] = None) -> List[int]:
+        """Token ids for logits [batch, vocab], as a list like the reference's sample()
+        (src/inference/model_runner.py:590-634); `sample_tokens` is the same without the copy to
+        the host."""
+        from .attention import sample_tokens
+        return sample_tokens(logits, temperature, top_p, uniforms).tolist()
+
     # ---------------------------------------------------------------- decode graphs
 
     @torch.inference_mode()

@@ -217,6 +217,34 @@ def fused_qk_times(pa, torch, dev, steps, warmup):
     return out
 
 
+def sampler_times(pa, torch, dev, steps, warmup):
+    """Token sampling for one decode step: 64 rows of 151 936 fp16 logits (Qwen3 vocabulary),
+    greedy and temperature 0.7 / top-p 0.9, beside the reference's sort-based procedure
+    (sort, softmax, cumsum, mask, scatter, softmax, multinomial) as torch ops on the same GPU."""
+    B, V = 64, 151936
+    g = torch.Generator(device=dev).manual_seed(9)
+    logits = (2.5 * torch.randn(B, V, generator=g, device=dev, dtype=torch.float32)).half()
+    u = torch.rand(B, generator=g, device=dev)
+
+    def reference_procedure():
+        scaled = logits.float() / 0.7
+        sl, si = torch.sort(scaled, descending=True, dim=-1)
+        cum = torch.cumsum(torch.softmax(sl, dim=-1), dim=-1)
+        mask = cum > 0.9
+        mask[..., 1:] = mask[..., :-1].clone()
+        mask[..., 0] = False
+        sl[mask] = float("-inf")
+        scaled = torch.zeros_like(scaled).scatter_(-1, si, sl)
+        return torch.multinomial(torch.softmax(scaled, dim=-1), num_samples=1).squeeze(-1)
+
+    ms_g, _ = time_steps(torch, lambda: pa.sample_tokens(logits, 0.0), steps, warmup)
+    ms_s, _ = time_steps(torch, lambda: pa.sample_tokens(logits, 0.7, 0.9, uniforms=u), steps, warmup)
+    ms_r, _ = time_steps(torch, reference_procedure, max(5, steps // 10), 2)
+    return {"workload": "64 x 151936 fp16 logits", "greedy_us": round(ms_g * 1e3, 1),
+            "top_p_us": round(ms_s * 1e3, 1), "sort_based_torch_us": round(ms_r * 1e3, 1),
+            "logit_bytes": B * V * 2}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -356,6 +384,7 @@ def main():
     line["prefill_mfma"] = prefill
     line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
     line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
+    line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))

@@ -228,6 +228,21 @@ int pa_qk_norm_rope_store(const void* q, const void* k, const void* v, int dtype
                           void* stream);
 
 /*
+ * One token per row of logits [batch, vocab] (f16 / bf16 / f32, rows row_stride elements apart),
+ * written to out [batch] (int64).
+ *   temperature <= 0: the index of the first maximum.
+ *   otherwise: p_i = softmax(logits / temperature); with top_p < 1 a token stays iff the mass of
+ *   the tokens with a strictly larger logit is <= top_p; the result is the first index j, in index
+ *   order over the kept tokens, whose running sum of p exceeds uniforms[row] * (kept mass).
+ *   uniforms: device fp32 [batch] in [0, 1), drawn by the caller (NULL allowed for greedy).
+ * No sort, no host synchronisation; the call can be captured in a graph.
+ * Replaces: ModelRunner.sample (src/inference/model_runner.py:590-634), whose multinomial draw is
+ * replaced by the inverse-CDF lookup with caller-supplied uniform numbers.
+ */
+int pa_sample(const void* logits, int dtype, int64_t row_stride, int64_t batch, int64_t vocab,
+              float temperature, float top_p, const float* uniforms, int64_t* out, void* stream);
+
+/*
  * Copy whole cache blocks inside one pool tensor laid out [num_planes][num_blocks][block_bytes]
  * (planes plane_stride_bytes apart): for every plane and every pair i, block pairs[2i+1] := block
  * pairs[2i].  The K/V tensor of a BlockPool is one such tensor with 2 x layers planes, each fp8
