@@ -121,7 +121,7 @@ def cpu_baseline(torch, w, scale, sample_seqs, bs, repeats=3):
 
 
 def prefill_cfg5a(pa, torch, dev, steps, warmup):
-    """BASELINE configs[4], first half: 8 sequences x (2048 cached + 512 new tokens), bf16 Q, FP16
+    """Fifth benchmark configuration, first half: 8 sequences x (2048 cached + 512 new tokens), bf16 Q, FP16
     KV, causal within the chunk; judged against the dense fp16 MFMA peak."""
     S, CACHED, NEW, HQ, HKV, D, BS = 8, 2048, 512, 16, 8, 128, 16
     g = torch.Generator(device=dev).manual_seed(1005)

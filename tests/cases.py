@@ -115,7 +115,7 @@ def uniform_lens(seed, batch, lo, hi):
     return torch.randint(lo, hi + 1, (batch,), generator=gen).tolist()
 
 
-# The five BASELINE configurations (decode side), by name.
+# The five benchmark configurations (decode side), by name.
 def config1(seed=1001):
     """bs 8, ctx U[128,512], pool of 512 blocks, fp16 KV."""
     return make_case(seed, uniform_lens(seed, 8, 128, 512), 512)

@@ -1,5 +1,5 @@
 """Paged decode attention on the GPU against the oracle (the reference's PyTorch paged
-attention restated on the CPU).  Tolerances are BASELINE's: rtol 1e-3 / atol 2e-3 for 16-bit
+attention restated on the CPU).  Tolerances are the ones stated for the path: rtol 1e-3 / atol 2e-3 for 16-bit
 caches, rtol 1e-2 / atol 1e-2 for fp8 caches."""
 import pytest
 import torch

@@ -1,6 +1,6 @@
 """Chunked-prefill paged attention (MFMA kernel) on the GPU against the oracle.
 
-fp16 / fp32 outputs use BASELINE's tolerances (rtol 1e-3 / atol 2e-3 for 16-bit caches,
+fp16 / fp32 outputs use the tolerances stated for the path (rtol 1e-3 / atol 2e-3 for 16-bit caches,
 1e-2 / 1e-2 for fp8).  bf16 outputs are compared with the oracle's unrounded fp32 result and
 are allowed one extra bf16 rounding (2^-8 relative) on top, since an 8-bit mantissa cannot
 resolve 1e-3.
