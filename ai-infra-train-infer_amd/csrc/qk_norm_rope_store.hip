@@ -11,7 +11,7 @@
 //
 // As separate ops that is some fourteen launches and six round trips of q and k through HBM per
 // layer; a decode step touches 64 tokens, so all of it is launch latency.  Here one workgroup
-// owns one token: each wave normalises and rotates whole head rows (a lane holds the rotation
+// (8 waves) owns one token: each wave normalises and rotates whole head rows (a lane holds the rotation
 // pair i, i + D/2, so the rotation needs no exchange), the rotated K row is collected in LDS so
 // that the fp8 writer can take its per-token amax over all heads, and K and V go to their cache
 // slot from there.  Intermediate roundings are those of the separate ops: the norm result is
@@ -49,6 +49,10 @@ struct NormRopeParams {
   float eps;
 };
 
+constexpr int kMaxRow = 4096;  // kv_heads * head_dim that fits the LDS staging row
+constexpr int kNormWaves = 8;  // waves per token: 24 head rows at the 16q/8kv shape, three per wave
+constexpr int kNormThreads = 64 * kNormWaves;
+
 __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
   if (dtype == PA_DTYPE_F16) return f16_bits_to_f32(f32_to_f16_bits(x));
   if (dtype == PA_DTYPE_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(x));
@@ -64,18 +68,30 @@ __device__ __forceinline__ float block_scale(float amax, float* red, int wave, i
   __syncthreads();                       // red may still be read from the previous use
   if (lane == 0) red[wave] = amax;
   __syncthreads();
-  amax = nan_keeping_max(nan_keeping_max(red[0], red[1]), nan_keeping_max(red[2], red[3]));
+  amax = red[0];
+#pragma unroll
+  for (int w = 1; w < kNormWaves; ++w) amax = nan_keeping_max(amax, red[w]);
   amax = amax < 1e-5f ? 1e-5f : amax;    // clamp(min=1e-5); NaN stays NaN
   return __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);   // torch: amax.reciprocal() * 448
 }
 
-constexpr int kMaxRow = 4096;  // kv_heads * head_dim that fits the LDS staging row
+
+// sin and cos of an fp32 angle that may be tens of thousands of radians (position x frequency).
+// The reduction to one revolution is done in fp64, where the product with 1/2pi is exact to far
+// below an fp32 ulp of the angle; the hardware sine / cosine then take the fraction of a turn.
+__device__ __forceinline__ void sincos_turns(float angle, float& sn, float& cs) {
+  double turns = (double)angle * 0.15915494309189535;
+  turns -= floor(turns);
+  const float f = (float)turns;
+  sn = __builtin_amdgcn_sinf(f);
+  cs = __builtin_amdgcn_cosf(f);
+}
 
 template <int D, bool FP8>
-__global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(const NormRopeParams p) {
+__global__ __launch_bounds__(kNormThreads) void qk_norm_rope_store_kernel(const NormRopeParams p) {
   constexpr int HALF = D / 2;
   __shared__ __align__(16) uint16_t krow[kMaxRow];   // rotated K of this token, activation dtype bits
-  __shared__ float red[4];
+  __shared__ float red[kNormWaves];
 
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63;
@@ -86,14 +102,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(const NormRopeP
 
   float cs, sn;
   {
-    const float angle = (float)p.positions[t] * p.inv_freq[i];
-    sn = sinf(angle);
-    cs = cosf(angle);
+    sincos_turns((float)p.positions[t] * p.inv_freq[i], sn, cs);
   }
   const float qw1 = load_as_f32(p.q_weight, i, p.weight_dtype), qw2 = load_as_f32(p.q_weight, i + HALF, p.weight_dtype);
   const float kw1 = load_as_f32(p.k_weight, i, p.weight_dtype), kw2 = load_as_f32(p.k_weight, i + HALF, p.weight_dtype);
 
-  for (int r = wave; r < p.hq + p.hkv; r += 4) {
+  for (int r = wave; r < p.hq + p.hkv; r += kNormWaves) {
     const bool is_k = r >= p.hq;
     const int head = is_k ? r - p.hq : r;
     const void* src = is_k ? p.k : p.q;
@@ -145,7 +159,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(const NormRopeP
     const int64_t row_bytes = (int64_t)row * es;
     uint8_t* kd = p.k_cache + slot * row_bytes;
     uint8_t* vd = p.v_cache + slot * row_bytes;
-    for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += 256 * 16) {
+    for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kNormThreads * 16) {
       *(uint4*)(kd + off) = *(const uint4*)((const uint8_t*)krow + off);
       *(uint4*)(vd + off) = *(const uint4*)(vsrc + off);
     }
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(const NormRopeP
     // quantising cache: per-token amax over all heads, scale = (1/amax) * 448, e4m3fn bytes
     auto quantise = [&](const void* src_row, uint8_t* dst, float* scale_dst) {
       float amax = 0.0f;
-      for (int e = threadIdx.x * 8; e < row; e += 256 * 8) {
+      for (int e = threadIdx.x * 8; e < row; e += kNormThreads * 8) {
         float x[8];
         load8_as_f32(src_row, e, p.dtype, x);
 #pragma unroll
@@ -161,7 +175,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(const NormRopeP
       }
       const float s = block_scale(amax, red, wave, lane);
       if (threadIdx.x == 0) *scale_dst = s;
-      for (int e = threadIdx.x * 8; e < row; e += 256 * 8) {
+      for (int e = threadIdx.x * 8; e < row; e += kNormThreads * 8) {
         float x[8];
         load8_as_f32(src_row, e, p.dtype, x);
         uint32_t w[2];
@@ -240,11 +254,11 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
   dim3 grid((unsigned)num_tokens);
   hipStream_t st = (hipStream_t)stream;
   if (head_dim == 128) {
-    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, true>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, false>), grid, dim3(256), 0, st, p);
+    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, true>), grid, dim3(kNormThreads), 0, st, p);
+    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, false>), grid, dim3(kNormThreads), 0, st, p);
   } else {
-    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, true>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, false>), grid, dim3(256), 0, st, p);
+    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, true>), grid, dim3(kNormThreads), 0, st, p);
+    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, false>), grid, dim3(kNormThreads), 0, st, p);
   }
   return check_launch("pa_qk_norm_rope_store");
 }

@@ -245,6 +245,45 @@ def sampler_times(pa, torch, dev, steps, warmup):
             "logit_bytes": B * V * 2}
 
 
+def model_step_cfg5b(pa, torch, dev, steps, warmup):
+    """Fifth benchmark configuration, second half: one decode step of a Qwen3-0.6B-shaped model
+    (28 layers, hidden 1024, 16q/8kv x 128, random weights) at batch 64, context 2048, FP16 KV:
+    metadata preparation + forward, eagerly and as a replayed HIP graph."""
+    cfg = pa.Qwen3PagedConfig()
+    B, CTX, BS = 64, 2048, 16
+    torch.manual_seed(11)
+    with torch.device(dev):
+        model = pa.Qwen3PagedModel(cfg).half().eval()
+    nb = B * (CTX // BS) + 8
+    pool = pa.BlockPool(nb, BS, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim, dtype=torch.float16, device=dev)
+    pool.kv_cache_tensor.normal_()
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(12))[:B * (CTX // BS)].view(B, -1)
+    seqs = [{"token_ids": [1] * CTX, "block_table": perm[b].tolist()} for b in range(B)]
+    out = {"workload": "Qwen3-0.6B shape, 28 layers, batch 64, ctx 2048, FP16 KV, one decode step"}
+    for name, graph in (("eager", False), ("hip_graph", True)):
+        runner = pa.ModelRunner(model, pa.ModelRunnerConfig(
+            num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
+            head_dim=cfg.head_dim, hidden_size=cfg.hidden_size, block_size=BS, max_num_blocks=CTX // BS,
+            device="cuda:0", enable_cuda_graph=graph, max_cuda_graph_batch_size=B))
+        runner.bind_kv_cache(pool.kv_cache_tensor)
+        if graph:
+            runner.capture_cuda_graphs([B])
+
+        def step():
+            ids, pos = runner.prepare_decode(seqs)
+            return runner.run(ids, pos, is_prefill=False)
+
+        ms, _ = time_steps(torch, step, steps, warmup)
+        out[name + "_ms"] = round(ms, 3)
+        runner.invalidate_cuda_graphs()
+    kv_bytes = cfg.num_layers * B * CTX * cfg.num_kv_heads * cfg.head_dim * 2 * 2
+    out["kv_bytes_per_step"] = kv_bytes
+    out["kv_gbps_in_graph_step"] = round(kv_bytes / out["hip_graph_ms"] / 1e6, 1)
+    del pool, model
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -385,6 +424,7 @@ def main():
     line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
     line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
     line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
+    line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
