@@ -293,6 +293,9 @@ def main():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=8)
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the auxiliary measurements (KV store, fused q/k kernel, sampler, model step): "
+                         "keeps a profiler trace of the run small")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device-to-device copies (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
@@ -421,10 +424,11 @@ def main():
         },
     }
     line["prefill_mfma"] = prefill
-    line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
-    line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
-    line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
-    line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
+    if not args.no_extras:
+        line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
+        line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
+        line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
+        line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
