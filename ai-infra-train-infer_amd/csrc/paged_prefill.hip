@@ -637,6 +637,8 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
     return fail(PA_ERR_UNSUPPORTED, "pa_prefill: fp8 K/V need the paged cache (block_tables)");
   if (head_dim != 64 && head_dim != 128)
     return fail(PA_ERR_UNSUPPORTED, "pa_prefill: head_dim must be 64 or 128");
+  if (!(scale > 0.0f) || scale > 3.0e38f)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: scale must be positive and finite (masked scores are -inf times scale)");
   if (num_q_heads % num_kv_heads != 0)
     return fail(PA_ERR_BAD_ARG, "pa_prefill: num_q_heads must be a multiple of num_kv_heads");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))

@@ -100,23 +100,34 @@ __global__ __launch_bounds__(kNormThreads) void qk_norm_rope_store_kernel(const 
   const bool active = lane < HALF;
   const int i = active ? lane : 0;
 
-  float cs, sn;
-  {
-    sincos_turns((float)p.positions[t] * p.inv_freq[i], sn, cs);
-  }
   const float qw1 = load_as_f32(p.q_weight, i, p.weight_dtype), qw2 = load_as_f32(p.q_weight, i + HALF, p.weight_dtype);
   const float kw1 = load_as_f32(p.k_weight, i, p.weight_dtype), kw2 = load_as_f32(p.k_weight, i + HALF, p.weight_dtype);
 
-  for (int r = wave; r < p.hq + p.hkv; r += kNormWaves) {
+  // Every head row of this wave is requested before any is worked on: the rows are independent
+  // and a wave that waits for one load at a time spends its life in memory latency.
+  constexpr int kRowsPerWave = 4;          // up to 32 head rows per token with 8 waves
+  const int nrows = p.hq + p.hkv;
+  float xa[kRowsPerWave], xb[kRowsPerWave];
+#pragma unroll
+  for (int j = 0; j < kRowsPerWave; ++j) {
+    const int r = wave + j * kNormWaves;
+    xa[j] = xb[j] = 0.0f;
+    if (active && r < nrows) {
+      const bool is_k = r >= p.hq;
+      const int64_t base = t * (is_k ? p.k_stride : p.q_stride) + (int64_t)(is_k ? r - p.hq : r) * D;
+      xa[j] = load_as_f32(is_k ? p.k : p.q, base + i, p.dtype);
+      xb[j] = load_as_f32(is_k ? p.k : p.q, base + i + HALF, p.dtype);
+    }
+  }
+  float cs, sn;
+  sincos_turns((float)p.positions[t] * p.inv_freq[i], sn, cs);
+#pragma unroll
+  for (int j = 0; j < kRowsPerWave; ++j) {
+    const int r = wave + j * kNormWaves;
+    if (r >= nrows) break;                 // wave-uniform
     const bool is_k = r >= p.hq;
     const int head = is_k ? r - p.hq : r;
-    const void* src = is_k ? p.k : p.q;
-    const int64_t base = t * (is_k ? p.k_stride : p.q_stride) + (int64_t)head * D;
-    float x1 = 0.0f, x2 = 0.0f;
-    if (active) {
-      x1 = load_as_f32(src, base + i, p.dtype);
-      x2 = load_as_f32(src, base + i + HALF, p.dtype);
-    }
+    const float x1 = xa[j], x2 = xb[j];
     float ss = x1 * x1 + x2 * x2;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
@@ -236,6 +247,8 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
       return fail(PA_ERR_BAD_ARG, "pa_qk_norm_rope_store: v rows and caches must be 16-byte aligned");
   }
   if (num_tokens > 0x7fffffff) return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: too many tokens");
+  if (num_q_heads + num_kv_heads > 4 * kNormWaves)
+    return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: more than 32 q + kv heads per token");
 
   NormRopeParams p;
   p.q = q; p.k = k; p.v = v;

@@ -178,6 +178,7 @@ int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* cont
  *                        K/V and Q are multiplied as fp16 with fp32 accumulation
  *   head_dim             64 or 128;  block_size a power of two
  *   max_seqlen_q         upper bound of Lq_s (sizes the launch grid)
+ *   scale                positive and finite
  */
 int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
@@ -213,7 +214,7 @@ int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
  *   pa_kv_store (kv_dtype == dtype) or pa_kv_store_fp8 (kv_dtype == PA_DTYPE_FP8_E4M3, per-token
  *   scales to k_scale / v_scale) would write them; slot < 0 or >= total_slots: no cache write.
  *   k_cache == NULL: no cache write at all (v, v_cache, scales, slot_mapping unused).
- * head_dim 64 or 128; Hkv * D * sizeof(dtype) <= 8192.
+ * head_dim 64 or 128; Hkv * D * sizeof(dtype) <= 8192; Hq + Hkv <= 32.
  * Replaces: RMSNorm.forward on q and k (src/distributed/tensor_parallel.py:78-84, used at
  * :453-454), _apply_rotary_emb (:394-419, used at :457-464) and store_kv_cache
  * (src/inference/attention.py:44-183) of one attention layer.

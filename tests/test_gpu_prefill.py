@@ -174,10 +174,12 @@ def test_waves_tunable_rejects_other_values(lib, gpu):
 def test_c_abi_argument_errors(lib, gpu):
     t = torch.zeros(64, dtype=torch.float16, device=gpu)
     p = t.data_ptr()
-    def call(d=128, hq=16, hkv=8, kvd=0, bt=p, bs=16):
+    def call(d=128, hq=16, hkv=8, kvd=0, bt=p, bs=16, scale=1.0):
         return lib.pa_prefill(p, 0, hq * d, p, p, None, None, kvd, bt, 4, p, p, p, hq * d, 1, 8, hq, hkv,
-                              d, bs, 4, 1.0, None)
+                              d, bs, 4, scale, None)
     assert call(d=96) == -2
     assert call(hq=15) == -1
     assert call(kvd=3) == -1
     assert call(bs=12) == -2
+    assert call(scale=0.0) == -1 and call(scale=-0.1) == -1 and call(scale=float("inf")) == -1
+    assert b"scale" in lib.pa_last_error()
