@@ -9,14 +9,16 @@
 // Here QK^T and PV are real dense tiles, so they run on v_mfma_f32_32x32x16_f16 with fp32
 // accumulation:
 //
-//  * One workgroup (4 waves) owns 128 query rows that share one KV head: 64 tokens x the two
-//    query heads of a GQA pair (or 128 tokens x 1 head).  Each wave owns 32 rows and keeps their
-//    Q as MFMA B operands in registers for the whole kernel.
+//  * One workgroup of W = 4 or 8 waves owns 32 W query rows that share one KV head: 16 W tokens x
+//    the two query heads of a GQA pair (or 32 W tokens x 1 head).  Each wave owns 32 rows and
+//    keeps their Q as MFMA B operands in registers for the whole kernel.  W = 8 puts twice the
+//    rows behind every K/V tile, which halves the bytes a CU pulls through its L1; large launches
+//    use it.
 //  * The KV sequence is walked in tiles of 64 keys.  A tile of K and of V (64 x head_dim) is
 //    fetched through the block table with 16-byte coalesced loads, converted to fp16 if the cache
 //    is bf16 / fp8 (fp8: value / per-token scale), and staged in LDS in its natural [key][dim]
 //    layout; LDS is double buffered so the loads of tile t+1 are in flight while tile t is
-//    multiplied.  All four waves read the same tile: every K/V byte is fetched once per 128 rows.
+//    multiplied.  All waves read the same tile: every K/V byte is fetched once per 32 W rows.
 //  * S^T = K . Q^T (keys x queries) rather than S: in the MFMA result layout a lane then holds 16
 //    keys of ONE query, so the online-softmax row max / row sum are in-lane reductions plus a
 //    single exchange with lane^32, and the fp16 probabilities are already laid out as the B
@@ -41,15 +43,6 @@ namespace pa {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
-typedef short short4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr;
-
-// LDS transpose load of gfx950: within each block of 16 lanes, lane i receives element (i % 4)
-// of the 8 bytes addressed by lanes 4j + i/4, j = 0..3 (checked on hardware).
-__device__ __forceinline__ half4_t lds_read_tr16(const _Float16* p) {
-  const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)p);
-  return __builtin_bit_cast(half4_t, r);
-}
 
 struct PrefillParams {
   const void* q;
@@ -77,18 +70,15 @@ enum : int { SRC_F16 = 0, SRC_BF16 = 1, SRC_FP8 = 2, SRC_F32 = 3 };
 
 constexpr int kBN = 64;  // keys per tile
 
-// One stage of a K or V tile in LDS: [key][head_dim] fp16 rows with no padding; the 16-byte
-// chunk c of row r lives at chunk position c ^ swz(r).  swz swaps the two low bit pairs of the
-// row number, so that (a) 16 consecutive rows get 16 different values: the 16 lanes that read
-// the same chunk index of 16 rows (MFMA A-operand reads of K) hit distinct banks, and (b) 4
-// consecutive rows differ in bits 2..3: the 4-row x 64-byte patch that 32 lanes fetch in one
-// pass of a transpose read of V spreads over 16 distinct chunk positions.
-// The same transpose read issued as opaque asm, for the tile loop of the fp16 path: the
-// compiler's wait-count pass cannot tell that the transpose-read builtin does not touch the buffer
-// that global_load_lds is filling, and drains every outstanding global load in front of it, in the
-// middle of the tile's arithmetic.  The result of an untracked read is not known to that pass
-// either: the caller waits with lds_wait<N> before use.  LDS operations complete in order, so the
-// extra outstanding reads only make the compiler's own lgkmcnt waits more conservative.
+// LDS reads of the tile loop, issued as opaque asm.  ds_read_b64_tr_b16 is the LDS transpose load
+// of gfx950: within each block of 16 lanes, lane i receives element (i % 4) of the 8 bytes
+// addressed by lanes 4j + i/4, j = 0..3 (checked on hardware).  Left to the compiler, every read
+// is followed by a wait and the product that uses it (ds_read -> s_waitcnt -> mfma, one k-step at a
+// time), and its wait-count pass, which cannot tell that a transpose read does not touch the
+// buffer that global_load_lds is filling, drains every outstanding global load in front of it.
+// The result of an untracked read is not known to that pass: the caller waits with lds_wait<N>
+// before use.  LDS operations complete in order, so the extra outstanding reads only make the
+// compiler's own lgkmcnt waits more conservative.
 template <int OFF>
 __device__ __forceinline__ half4_t tr_read_untracked(uint32_t lds_byte_addr) {
   half4_t r;
@@ -122,6 +112,12 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// One stage of a K or V tile in LDS: [key][head_dim] fp16 rows with no padding; the 16-byte
+// chunk c of row r lives at chunk position c ^ swz(r).  swz swaps the two low bit pairs of the
+// row number, so that (a) 16 consecutive rows get 16 different values: the 16 lanes that read
+// the same chunk index of 16 rows (MFMA A-operand reads of K) hit distinct banks, and (b) 4
+// consecutive rows differ in bits 2..3: the 4-row x 64-byte patch that 32 lanes fetch in one
+// pass of a transpose read of V spreads over 16 distinct chunk positions.
 template <int CPR>
 __device__ __forceinline__ constexpr int swz(int row) {
   return (((row & 3) << 2) | ((row >> 2) & 3)) & (CPR - 1);
@@ -171,10 +167,11 @@ __device__ __forceinline__ half8_t load8_as_f16(const uint8_t* p, float inv_scal
 template <int SRC>
 constexpr int src_bytes() { return SRC == SRC_FP8 ? 1 : (SRC == SRC_F32 ? 4 : 2); }
 
-// DIRECT: fp16 sources go global -> LDS with global_load_lds_dwordx4 (no staging registers, two
-// workgroups per CU); other source types are converted in registers on the way (one per CU).
+// DIRECT: fp16 sources go global -> LDS with global_load_lds_dwordx4 (no staging registers); other
+// source types are converted in registers on the way.  W = waves per workgroup: 4 (two workgroups
+// per CU) or 8 (one, with twice the query rows behind every K/V tile).
 template <int D, int HPWG, int SRC, int W>
-__global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void paged_prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel(const PrefillParams p) {
   constexpr int NT = 64 * W;              // threads per workgroup
   using L = PrefillLds<D>;
   constexpr bool DIRECT = SRC == SRC_F16;
@@ -253,7 +250,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
   // ---- staging: global -> (registers ->) LDS ---------------------------------------------------------
   // chunk = 16 bytes of fp16 = 8 head-dim elements; thread `tid` moves chunks tid, tid+NT, ...
   // i.e. one instruction of a wave covers 64 / CPR whole rows, contiguous in LDS.
-  auto row_slot = [&](int key) -> int64_t {   // physical row of a key (clamped: never faults)
+  auto row_slot = [&](int key) __attribute__((always_inline)) -> int64_t {   // physical row of a key (clamped: never faults)
     const int kk = min(key, lk - 1);
     if (bt_row) {
       const int blk = min(kk >> p.bs_log2, bt_last);
@@ -276,7 +273,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
     const int col = (chunk % CPR) ^ swz<CPR>(row);
     lane_part[c] = (uint32_t)(((lane / CPR) * token_elems + (int64_t)kvh * D + col * 8) * ES);
   }
-  auto move_chunk = [&](int c, int buf, const uint8_t* kp, const uint8_t* vp, int64_t slot) {
+  auto move_chunk = [&](int c, int buf, const uint8_t* kp, const uint8_t* vp, int64_t slot) __attribute__((always_inline)) {
     if constexpr (DIRECT) {
       const int wbase = (NT * c + (tid & ~63)) * 8;   // LDS destination = wave base + lane * 16 bytes
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
@@ -295,12 +292,12 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
   };
   // Block-table entries of a tile, fetched one tile ahead of the loads that need them so that no
   // load ever waits on another: lane l holds the entry of chunk group l % NCH of this wave.
-  auto load_ids = [&](int t) -> int {
+  auto load_ids = [&](int t) __attribute__((always_inline)) -> int {
     if (!bt_row) return 0;
     const int row0 = (NT * (lane % NCH) + 64 * wave) / CPR;
     return bt_row[min((t * kBN + row0) >> p.bs_log2, bt_last)];
   };
-  auto fetch = [&](int t, int buf, int ids) {
+  auto fetch = [&](int t, int buf, int ids) __attribute__((always_inline)) {
     if (uniform_rows && (t + 1) * kBN <= lk) {
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
@@ -328,7 +325,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
       move_chunk(c, buf, p.k + eoff, p.v + eoff, slot);
     }
   };
-  auto commit = [&](int buf) {
+  auto commit = [&](int buf) __attribute__((always_inline)) {
     if constexpr (!DIRECT) {
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
@@ -373,7 +370,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
 
   // `buf` is a compile-time constant (the tile loop is unrolled by two) so that every LDS read
   // below is "loop-invariant register + immediate offset".
-  auto compute = [&](int t, auto buf_tag) {
+  auto compute = [&](int t, auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
     const int kt0 = t * kBN;
     // ---- S^T = K . Q^T : two 32-key tiles -------------------------------------------------------
@@ -382,36 +379,26 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
-    if constexpr (DIRECT) {
-      // All K fragments of the first 32-key half are requested at once and those of the second
-      // half as the first are consumed, so a product never waits for a read issued just before it.
-      constexpr int OFF0 = buf * kBN * D * 2, OFF1 = OFF0 + 32 * D * 2;
-      half8_t ka[KSTEPS], kb[KSTEPS];
+    // All K fragments of the first 32-key half are requested at once and those of the second
+    // half as the first are consumed, so a product never waits for a read issued just before it.
+    constexpr int OFF0 = buf * kBN * D * 2, OFF1 = OFF0 + 32 * D * 2;
+    half8_t ka[KSTEPS], kb[KSTEPS];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) ka[ks] = b128_read_untracked<OFF0>(k_addr[ks]);
-      static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
-        constexpr int ks = 2 * decltype(j_tag)::value;
-        lds_wait<KSTEPS - 2>(ka[ks], ka[ks + 1]);   // outstanding: the rest of ka and what is issued of kb
-        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks], qreg[ks], s[0], 0, 0, 0);
-        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks + 1], qreg[ks + 1], s[0], 0, 0, 0);
-        kb[ks] = b128_read_untracked<OFF1>(k_addr[ks]);
-        kb[ks + 1] = b128_read_untracked<OFF1>(k_addr[ks + 1]);
-      });
-      static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
-        constexpr int ks = 2 * decltype(j_tag)::value;
-        lds_wait<KSTEPS - 2 - ks>(kb[ks], kb[ks + 1]);
-        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks], qreg[ks], s[1], 0, 0, 0);
-        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks + 1], qreg[ks + 1], s[1], 0, 0, 0);
-      });
-    } else {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const half8_t a = *(const half8_t*)&lds.k[buf][kt * 32 * D + k_off[ks]];
-          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], s[kt], 0, 0, 0);
-        }
-    }
+    for (int ks = 0; ks < KSTEPS; ++ks) ka[ks] = b128_read_untracked<OFF0>(k_addr[ks]);
+    static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
+      constexpr int ks = 2 * decltype(j_tag)::value;
+      lds_wait<KSTEPS - 2>(ka[ks], ka[ks + 1]);   // outstanding: the rest of ka and what is issued of kb
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks], qreg[ks], s[0], 0, 0, 0);
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks + 1], qreg[ks + 1], s[0], 0, 0, 0);
+      kb[ks] = b128_read_untracked<OFF1>(k_addr[ks]);
+      kb[ks + 1] = b128_read_untracked<OFF1>(k_addr[ks + 1]);
+    });
+    static_for<KSTEPS / 2>([&](auto j_tag) __attribute__((always_inline)) {
+      constexpr int ks = 2 * decltype(j_tag)::value;
+      lds_wait<KSTEPS - 2 - ks>(kb[ks], kb[ks + 1]);
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks], qreg[ks], s[1], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb[ks + 1], qreg[ks + 1], s[1], 0, 0, 0);
+    });
     // ---- mask: only tiles that reach past the diagonal of this wave or the sequence end ---------
     const int wave_first_lim = tokw0 + shift;  // smallest row limit in the wave
     if (kt0 + kBN - 1 > wave_first_lim || kt0 + kBN > lk) {
@@ -461,58 +448,43 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
       }
     l_run += psum;
     // ---- O^T += V^T . P^T : four 16-key steps x MT row tiles ----------------------------------------
-    if constexpr (DIRECT) {
-      // untracked reads, one 16-key step ahead of the products that use them
-      half4_t lo[2][MT], hi[2][MT];
-      auto issue = [&](auto k2_tag) __attribute__((always_inline)) {
-        constexpr int k2 = decltype(k2_tag)::value;
-        constexpr int OFF = (buf * kBN * D + k2 * 16 * D) * 2;
+    // untracked reads, one 16-key step ahead of the products that use them
+    half4_t lo[2][MT], hi[2][MT];
+    auto issue = [&](auto k2_tag) __attribute__((always_inline)) {
+      constexpr int k2 = decltype(k2_tag)::value;
+      constexpr int OFF = (buf * kBN * D + k2 * 16 * D) * 2;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          lo[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][0]);
-          hi[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][1]);
-        }
-      };
-      auto multiply = [&](auto k2_tag) __attribute__((always_inline)) {
-        constexpr int k2 = decltype(k2_tag)::value;
-        // reads return in order: this step's have all landed once no more than the next step's
-        // 2 MT are outstanding.  volatile asm statements keep their order, so tying the other
-        // registers to empty statements after the wait holds their consumers below it too.
-        if constexpr (k2 < 3) lds_wait<2 * MT>(lo[k2 & 1][0], hi[k2 & 1][0]);
-        else lds_wait<0>(lo[k2 & 1][0], hi[k2 & 1][0]);
-#pragma unroll
-        for (int mt = 1; mt < MT; ++mt) asm volatile("" : "+v"(lo[k2 & 1][mt]), "+v"(hi[k2 & 1][mt]));
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const half4_t l4 = lo[k2 & 1][mt], h4 = hi[k2 & 1][mt];
-          half8_t a;
-          a[0] = l4[0]; a[1] = l4[1]; a[2] = l4[2]; a[3] = l4[3];
-          a[4] = h4[0]; a[5] = h4[1]; a[6] = h4[2]; a[7] = h4[3];
-          o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
-        }
-      };
-      issue(std::integral_constant<int, 0>{});
-      issue(std::integral_constant<int, 1>{});
-      multiply(std::integral_constant<int, 0>{});
-      issue(std::integral_constant<int, 2>{});
-      multiply(std::integral_constant<int, 1>{});
-      issue(std::integral_constant<int, 3>{});
-      multiply(std::integral_constant<int, 2>{});
-      multiply(std::integral_constant<int, 3>{});
-    } else {
-#pragma unroll
-      for (int k2 = 0; k2 < 4; ++k2) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const half4_t lo = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][0]]);
-          const half4_t hi = lds_read_tr16(&lds.v[buf][k2 * 16 * D + v_off[mt][1]]);
-          half8_t a;
-          a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
-          a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
-          o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
-        }
+      for (int mt = 0; mt < MT; ++mt) {
+        lo[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][0]);
+        hi[k2 & 1][mt] = tr_read_untracked<OFF>(v_addr[mt][1]);
       }
-    }
+    };
+    auto multiply = [&](auto k2_tag) __attribute__((always_inline)) {
+      constexpr int k2 = decltype(k2_tag)::value;
+      // reads return in order: this step's have all landed once no more than the next step's
+      // 2 MT are outstanding.  volatile asm statements keep their order, so tying the other
+      // registers to empty statements after the wait holds their consumers below it too.
+      if constexpr (k2 < 3) lds_wait<2 * MT>(lo[k2 & 1][0], hi[k2 & 1][0]);
+      else lds_wait<0>(lo[k2 & 1][0], hi[k2 & 1][0]);
+#pragma unroll
+      for (int mt = 1; mt < MT; ++mt) asm volatile("" : "+v"(lo[k2 & 1][mt]), "+v"(hi[k2 & 1][mt]));
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const half4_t l4 = lo[k2 & 1][mt], h4 = hi[k2 & 1][mt];
+        half8_t a;
+        a[0] = l4[0]; a[1] = l4[1]; a[2] = l4[2]; a[3] = l4[3];
+        a[4] = h4[0]; a[5] = h4[1]; a[6] = h4[2]; a[7] = h4[3];
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[k2], o[mt], 0, 0, 0);
+      }
+    };
+    issue(std::integral_constant<int, 0>{});
+    issue(std::integral_constant<int, 1>{});
+    multiply(std::integral_constant<int, 0>{});
+    issue(std::integral_constant<int, 2>{});
+    multiply(std::integral_constant<int, 1>{});
+    issue(std::integral_constant<int, 3>{});
+    multiply(std::integral_constant<int, 2>{});
+    multiply(std::integral_constant<int, 3>{});
   };
 
   // ---- tile loop: LDS double buffer, one barrier per tile -------------------------------------------
@@ -524,7 +496,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 && SRC == SRC_F16 ? 2 : 1)) void pa
     if (ntiles > 1) ids = load_ids(1);
   }
   __syncthreads();
-  auto step = [&](int t, auto buf_tag) {
+  auto step = [&](int t, auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
     if (t + 1 < ntiles) {
       fetch(t + 1, buf ^ 1, ids);      // direct loads land in the other buffer while this one is used
