@@ -488,12 +488,18 @@ class PartitionedPagedAttention(PagedAttention):
     The reference picks the path after a host read of max(context_lens); here the launch is
     sized from the block-table width instead, so no host synchronisation happens: sequences
     shorter than one partition simply own a single partition, which merges to itself.
+
+    partition_size is the finest split the layer will use.  The merge is exact, so when the
+    batch already fills the GPU with coarser partitions (or with none) the launch takes those:
+    at 256 sequences a split into 512-token partitions only adds partial results to write and
+    merge.  `adaptive = False` keeps every launch at exactly partition_size.
     """
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int,
                  cache_dtype: str = "fp16", partition_size: int = 512):
         super().__init__(num_heads, num_kv_heads, head_dim, cache_dtype)
         self.partition_size = partition_size
+        self.adaptive = True
 
     def _decode_attention(self, q, ctx):
         if ctx.context_lens is None:
@@ -504,6 +510,12 @@ class PartitionedPagedAttention(PagedAttention):
         if self.k_cache is None or ctx.block_tables is None or ctx.context_lens is None:
             return q
         ks, vs = self._scales()
+        psize = self.partition_size
+        if self.adaptive:
+            max_context = ctx.block_tables.shape[1] * self.k_cache.shape[1]
+            auto, _ = choose_partition(q.shape[0], self.num_heads, self.num_kv_heads, max_context,
+                                       self.head_dim, self.k_cache.element_size())
+            if auto == 0 or auto >= psize:
+                psize = None          # the launch's own choice: single pass or coarser partitions
         return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
-                            self.scale, k_scale=ks, v_scale=vs,
-                            partition_size=self.partition_size)
+                            self.scale, k_scale=ks, v_scale=vs, partition_size=psize)

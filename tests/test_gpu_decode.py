@@ -227,3 +227,19 @@ def test_c_abi_argument_errors(lib, gpu):
     assert call(kvd=3) == -1                      # fp8 without scales
     assert call(parts=4, psize=500, ws=p, wsb=1 << 30) == -2      # not a multiple of 16
     assert call(parts=4, psize=512) == -4         # workspace missing
+
+
+@pytest.mark.parametrize("adaptive", [True, False])
+def test_partitioned_module_adaptive_and_exact_splits_agree(pa, gpu, adaptive):
+    # long contexts at a small batch (split finer than the layer's size is never used) and a large
+    # batch (no split needed): the layer's answer does not depend on how the launch was cut
+    for seed, lens in ((50, [3000, 5000, 4097, 700]), (51, [300] * 130)):
+        c = cases.make_case(seed, lens, sum((l + 15) // 16 for l in lens) + 8)
+        d = cases.to_device(c, gpu)
+        attn = pa.PartitionedPagedAttention(16, 8, 128, partition_size=512)
+        attn.adaptive = adaptive
+        attn.k_cache, attn.v_cache = d["k_cache"], d["v_cache"]
+        pa.set_context(False, context_lens=d["context_lens"], block_tables=d["block_tables"])
+        got = attn._decode_attention(d["q"], pa.get_context()).cpu()
+        pa.reset_context()
+        check(got, oracle_decode(c), "fp16")
