@@ -171,8 +171,15 @@ def qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, pos
     hkv = k.shape[1]
     if k.dtype != q.dtype or (v is not None and v.dtype != q.dtype):
         raise RuntimeError("qk_norm_rope_store: q, k and v dtypes differ")
-    q, qs = _rows(q, "qk_norm_rope_store")
-    k, ks_ = _rows(k, "qk_norm_rope_store")
+    def rows16(t):
+        """rows as the kernel moves them: 16-byte pieces"""
+        t, stride = _rows(t, "qk_norm_rope_store")
+        if t.data_ptr() % 16 or (stride * t.element_size()) % 16:
+            t = t.contiguous()
+            stride = t.shape[1] * t.shape[2]
+        return t, stride
+    q, qs = rows16(q)
+    k, ks_ = rows16(k)
     if q_norm_weight.numel() != d or k_norm_weight.numel() != d or q_norm_weight.dtype != k_norm_weight.dtype:
         raise RuntimeError("qk_norm_rope_store: norm weights must both be [head_dim] of one dtype")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() != d // 2:
@@ -191,7 +198,7 @@ def qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, pos
         if tuple(k_cache.shape[2:]) != (hkv, d) or v is None or v.shape != k.shape:
             raise RuntimeError("qk_norm_rope_store: k/v %s do not match the cache %s"
                                % (tuple(k.shape), tuple(k_cache.shape)))
-        v, vs_ = _rows(v, "qk_norm_rope_store")
+        v, vs_ = rows16(v)
         total_slots = k_cache.shape[0] * k_cache.shape[1]
         if slot_mapping.numel() != n:
             raise RuntimeError("qk_norm_rope_store: slot_mapping has %d entries for %d tokens"

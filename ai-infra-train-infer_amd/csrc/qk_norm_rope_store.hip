@@ -10,13 +10,14 @@
 //     store_kv_cache(k, v, k_cache, v_cache, slot_mapping, ...)
 //
 // As separate ops that is some fourteen launches and six round trips of q and k through HBM per
-// layer; a decode step touches 64 tokens, so all of it is launch latency.  Here one workgroup
-// (8 waves) owns one token: each wave normalises and rotates whole head rows (a lane holds the rotation
-// pair i, i + D/2, so the rotation needs no exchange), the rotated K row is collected in LDS so
-// that the fp8 writer can take its per-token amax over all heads, and K and V go to their cache
-// slot from there.  Intermediate roundings are those of the separate ops: the norm result is
-// rounded to the activation dtype, the rotation is done in fp32 on that and rounded again, and
-// the fp8 writer sees exactly the values a separate store would see.
+// layer; a decode step touches 64 tokens, so all of it is launch latency.  Here one wave owns
+// one token and nothing leaves its registers: a lane holds 8 consecutive elements of a head row
+// (16-byte accesses; 16 lanes per row at head_dim 128, so one instruction covers four heads), the
+// rotation partner of an element sits 8 lanes away (one cross-lane move), RMSNorm needs a
+// 16-lane sum, and the per-token amax of the fp8 writer is a wave reduction over the rotated K
+// rows the wave still holds.  Intermediate roundings are those of the separate ops: the norm
+// result is rounded to the activation dtype, the rotation is done in fp32 on that and rounded
+// again, and the fp8 writer sees exactly the values a separate store would see.
 #include "pa_common.hpp"
 #include "pa_host.hpp"
 
@@ -43,15 +44,15 @@ struct NormRopeParams {
   float* v_scale;
   const int32_t* slot_mapping;
   int64_t total_slots;
+  int64_t num_tokens;
   int dtype;                              // q, k, v, q_out, k_out (and the cache, unless fp8)
   int weight_dtype;
   int hq, hkv;
   float eps;
 };
 
-constexpr int kMaxRow = 4096;  // kv_heads * head_dim that fits the LDS staging row
-constexpr int kNormWaves = 8;  // waves per token: 24 head rows at the 16q/8kv shape, three per wave
-constexpr int kNormThreads = 64 * kNormWaves;
+constexpr int kTokensPerGroup = 4;   // waves (= tokens) per workgroup
+constexpr int kMaxKvGroups = 4;      // K row groups a wave keeps in registers: kv_heads * head_dim <= 2048
 
 __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
   if (dtype == PA_DTYPE_F16) return f16_bits_to_f32(f32_to_f16_bits(x));
@@ -60,21 +61,6 @@ __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
 }
 
 __device__ __forceinline__ float nan_keeping_max(float m, float a) { return (a > m || a != a) ? a : m; }
-
-// amax of the workgroup's values -> clamp -> scale, as the quantising store computes them
-__device__ __forceinline__ float block_scale(float amax, float* red, int wave, int lane) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) amax = nan_keeping_max(amax, __shfl_xor(amax, o));
-  __syncthreads();                       // red may still be read from the previous use
-  if (lane == 0) red[wave] = amax;
-  __syncthreads();
-  amax = red[0];
-#pragma unroll
-  for (int w = 1; w < kNormWaves; ++w) amax = nan_keeping_max(amax, red[w]);
-  amax = amax < 1e-5f ? 1e-5f : amax;    // clamp(min=1e-5); NaN stays NaN
-  return __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);   // torch: amax.reciprocal() * 448
-}
-
 
 // sin and cos of an fp32 angle that may be tens of thousands of radians (position x frequency).
 // The reduction to one revolution is done in fp64, where the product with 1/2pi is exact to far
@@ -87,121 +73,185 @@ __device__ __forceinline__ void sincos_turns(float angle, float& sn, float& cs) 
   cs = __builtin_amdgcn_cosf(f);
 }
 
-template <int D, bool FP8>
-__global__ __launch_bounds__(kNormThreads) void qk_norm_rope_store_kernel(const NormRopeParams p) {
-  constexpr int HALF = D / 2;
-  __shared__ __align__(16) uint16_t krow[kMaxRow];   // rotated K of this token, activation dtype bits
-  __shared__ float red[kNormWaves];
+// eight consecutive elements (index i a multiple of 8, 16-byte aligned rows) from fp32
+__device__ __forceinline__ void store8_from_f32(void* p, int64_t i, int dtype, const float (&x)[8]) {
+  if (dtype == PA_DTYPE_F32) {
+    *(float4*)((float*)p + i) = make_float4(x[0], x[1], x[2], x[3]);
+    *(float4*)((float*)p + i + 4) = make_float4(x[4], x[5], x[6], x[7]);
+  } else {
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = dtype == PA_DTYPE_F16 ? f32_to_f16_bits(x[2 * k]) : f32_to_bf16_bits(x[2 * k]);
+      const uint32_t hi = dtype == PA_DTYPE_F16 ? f32_to_f16_bits(x[2 * k + 1]) : f32_to_bf16_bits(x[2 * k + 1]);
+      w[k] = lo | (hi << 16);
+    }
+    *(uint4*)((uint16_t*)p + i) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
 
-  const int64_t t = blockIdx.x;
+// amax over the wave -> clamp -> scale, as the quantising store computes them
+__device__ __forceinline__ float wave_scale(float amax) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = nan_keeping_max(amax, __shfl_xor(amax, o));
+  amax = amax < 1e-5f ? 1e-5f : amax;    // clamp(min=1e-5); NaN stays NaN
+  return __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);   // torch: amax.reciprocal() * 448
+}
+
+__device__ __forceinline__ uint2 encode8(const float (&x)[8], float s) {
+  uint32_t w[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    uint32_t b = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) b |= f32_to_e4m3fn(__fmul_rn(x[4 * j + k], s)) << (8 * k);
+    w[j] = b;
+  }
+  return make_uint2(w[0], w[1]);
+}
+
+// DT = activation dtype, a template parameter: a run-time switch inside every 8-element load and
+// store would put a branch (and a wait) between the loads that are meant to be in flight together.
+template <int D, bool FP8, int DT>
+__global__ __launch_bounds__(64 * kTokensPerGroup) void qk_norm_rope_store_kernel(const NormRopeParams p) {
+  constexpr int LPR = D / 8;          // lanes per head row
+  constexpr int RPI = 64 / LPR;       // head rows per wave instruction
+  constexpr int PAIR = LPR / 2;       // lane distance to the rotation partner
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int es = p.dtype == PA_DTYPE_F32 ? 4 : 2;
-  const bool active = lane < HALF;
-  const int i = active ? lane : 0;
+  const int64_t t = (int64_t)blockIdx.x * kTokensPerGroup + (threadIdx.x >> 6);
+  if (t >= p.num_tokens) return;      // the whole wave
+  const int c = lane % LPR;           // which 8 elements of the row
+  const int sub = lane / LPR;         // which row of the group
+  const bool upper = c >= PAIR;       // second half of the row
+  const int f0 = (c % PAIR) * 8;      // first of this lane's 8 frequencies
 
-  const float qw1 = load_as_f32(p.q_weight, i, p.weight_dtype), qw2 = load_as_f32(p.q_weight, i + HALF, p.weight_dtype);
-  const float kw1 = load_as_f32(p.k_weight, i, p.weight_dtype), kw2 = load_as_f32(p.k_weight, i + HALF, p.weight_dtype);
-
-  // Every head row of this wave is requested before any is worked on: the rows are independent
+  // loads first, all of them: position, frequencies, weights and (below) every row of the token
+  const float pos = (float)p.positions[t];
+  const float4 fa = *(const float4*)(p.inv_freq + f0), fb = *(const float4*)(p.inv_freq + f0 + 4);
+  float qw[8], kw[8];
+  load8_as_f32(p.q_weight, c * 8, p.weight_dtype, qw);
+  load8_as_f32(p.k_weight, c * 8, p.weight_dtype, kw);
+  // Every row group of the token is requested before any is worked on: they are independent,
   // and a wave that waits for one load at a time spends its life in memory latency.
-  constexpr int kRowsPerWave = 4;          // up to 32 head rows per token with 8 waves
-  const int nrows = p.hq + p.hkv;
-  float xa[kRowsPerWave], xb[kRowsPerWave];
+  constexpr int kQGroupsAhead = 4;      // q row groups loaded up front (16 heads at head_dim 128)
+  float qx[kQGroupsAhead][8], kx[kMaxKvGroups][8], vx[kMaxKvGroups][8];
 #pragma unroll
-  for (int j = 0; j < kRowsPerWave; ++j) {
-    const int r = wave + j * kNormWaves;
-    xa[j] = xb[j] = 0.0f;
-    if (active && r < nrows) {
-      const bool is_k = r >= p.hq;
-      const int64_t base = t * (is_k ? p.k_stride : p.q_stride) + (int64_t)(is_k ? r - p.hq : r) * D;
-      xa[j] = load_as_f32(is_k ? p.k : p.q, base + i, p.dtype);
-      xb[j] = load_as_f32(is_k ? p.k : p.q, base + i + HALF, p.dtype);
+  for (int g = 0; g < kQGroupsAhead; ++g) {
+    const int head = g * RPI + sub;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qx[g][e] = 0.0f;
+    if (head < p.hq) load8_as_f32(p.q, t * p.q_stride + (int64_t)head * D + c * 8, DT, qx[g]);
+  }
+  const bool write = p.k_cache != nullptr;
+  const int64_t slot = write ? (int64_t)p.slot_mapping[t] : -1;
+#pragma unroll
+  for (int g = 0; g < kMaxKvGroups; ++g) {
+    const int head = g * RPI + sub;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) kx[g][e] = vx[g][e] = 0.0f;
+    if (head < p.hkv) {
+      load8_as_f32(p.k, t * p.k_stride + (int64_t)head * D + c * 8, DT, kx[g]);
+      if (write) load8_as_f32(p.v, t * p.v_stride + (int64_t)head * D + c * 8, DT, vx[g]);
     }
   }
-  float cs, sn;
-  sincos_turns((float)p.positions[t] * p.inv_freq[i], sn, cs);
+
+  float cs[8], sn[8];
+  {
+    const float fr[8] = {fa.x, fa.y, fa.z, fa.w, fb.x, fb.y, fb.z, fb.w};
 #pragma unroll
-  for (int j = 0; j < kRowsPerWave; ++j) {
-    const int r = wave + j * kNormWaves;
-    if (r >= nrows) break;                 // wave-uniform
-    const bool is_k = r >= p.hq;
-    const int head = is_k ? r - p.hq : r;
-    const float x1 = xa[j], x2 = xb[j];
-    float ss = x1 * x1 + x2 * x2;
+    for (int e = 0; e < 8; ++e) sincos_turns(pos * fr[e], sn[e], cs[e]);
+  }
+
+  // x: this lane's 8 elements of a head row -> normalised, rounded, rotated, rounded (as fp32)
+  auto norm_rope = [&](float (&x)[8], const float (&w)[8]) __attribute__((always_inline)) {
+    float ss = 0.0f;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-    const float inv = rsqrtf(ss / (float)D + p.eps);
-    // the norm returns the activation dtype; the rotation then works in fp32 on those values
-    const float y1 = round_to_dtype((is_k ? kw1 : qw1) * (x1 * inv), p.dtype);
-    const float y2 = round_to_dtype((is_k ? kw2 : qw2) * (x2 * inv), p.dtype);
-    const float o1 = y1 * cs + (-y2) * sn;
-    const float o2 = y2 * cs + y1 * sn;
-    if (!active) continue;
-    if (!is_k) {
-      const int64_t ob = t * p.q_out_stride + (int64_t)head * D;
-      store_from_f32(p.q_out, ob + i, p.dtype, o1);
-      store_from_f32(p.q_out, ob + i + HALF, p.dtype, o2);
+    for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+    // sum over the LPR lanes of the row, by lane-permute moves inside a 16-lane row
+    ss += dpp_f32<0xB1>(ss);                        // quad_perm [1,0,3,2]
+    ss += dpp_f32<0x4E>(ss);                        // quad_perm [2,3,0,1]
+    if constexpr (LPR == 16) {
+      ss += dpp_f32<0x124>(ss);                     // row_ror:4
+      ss += dpp_f32<0x128>(ss);                     // row_ror:8
     } else {
-      if (p.k_out) {
-        const int64_t ob = t * p.k_out_stride + (int64_t)head * D;
-        store_from_f32(p.k_out, ob + i, p.dtype, o1);
-        store_from_f32(p.k_out, ob + i + HALF, p.dtype, o2);
-      }
-      if (p.dtype == PA_DTYPE_F32) {
-        ((float*)krow)[head * D + i] = o1;          // fp32 activations: the row is kMaxRow / 2 long at most
-        ((float*)krow)[head * D + i + HALF] = o2;
-      } else {
-        krow[head * D + i] = p.dtype == PA_DTYPE_F16 ? f32_to_f16_bits(o1) : f32_to_bf16_bits(o1);
-        krow[head * D + i + HALF] = p.dtype == PA_DTYPE_F16 ? f32_to_f16_bits(o2) : f32_to_bf16_bits(o2);
-      }
+      ss += dpp_f32<0x141>(ss);                     // row_half_mirror: lane i <-> 7 - i
+    }
+    const float inv = rsqrtf(ss / (float)D + p.eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      // the norm returns the activation dtype; the rotation then works in fp32 on those values
+      const float y = round_to_dtype(w[e] * (x[e] * inv), DT);
+      // the rotation partner: 8 lanes away in a 16-lane row (row_ror:8), 4 away in an 8-lane one
+      const float other = LPR == 16 ? dpp_f32<0x128>(y) : __shfl_xor(y, PAIR);
+      const float rotated = upper ? other : -other;      // cat(-x2, x1)
+      x[e] = round_to_dtype(y * cs[e] + rotated * sn[e], DT);
+    }
+  };
+
+  // ---- q ------------------------------------------------------------------------------------------
+#pragma unroll
+  for (int g = 0; g < kQGroupsAhead; ++g) {
+    const int head = g * RPI + sub;
+    if (g * RPI < p.hq) {                // wave-uniform
+      norm_rope(qx[g], qw);
+      if (head < p.hq) store8_from_f32(p.q_out, t * p.q_out_stride + (int64_t)head * D + c * 8, DT, qx[g]);
     }
   }
-  __syncthreads();
+  for (int g = kQGroupsAhead; g * RPI < p.hq; ++g) {      // more query heads than were loaded up front
+    const int head = g * RPI + sub;
+    const bool live = head < p.hq;
+    float x[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (live) load8_as_f32(p.q, t * p.q_stride + (int64_t)head * D + c * 8, DT, x);
+    norm_rope(x, qw);
+    if (live) store8_from_f32(p.q_out, t * p.q_out_stride + (int64_t)head * D + c * 8, DT, x);
+  }
 
-  if (!p.k_cache) return;
-  const int64_t slot = p.slot_mapping[t];
-  if (slot < 0 || slot >= p.total_slots) return;   // uniform over the workgroup
-  const int row = p.hkv * D;
-  const uint8_t* vsrc = (const uint8_t*)p.v + t * p.v_stride * es;
+  // ---- k: the rotated rows stay in registers for the cache write -------------------------------------
+#pragma unroll
+  for (int g = 0; g < kMaxKvGroups; ++g) {
+    const int head = g * RPI + sub;
+    if (g * RPI < p.hkv) {               // wave-uniform
+      norm_rope(kx[g], kw);
+      if (head < p.hkv && p.k_out)
+        store8_from_f32(p.k_out, t * p.k_out_stride + (int64_t)head * D + c * 8, DT, kx[g]);
+    }
+  }
 
+  // ---- cache write ----------------------------------------------------------------------------------
+  if (!write || slot < 0 || slot >= p.total_slots) return;   // uniform over the wave
+  const int64_t row = (int64_t)p.hkv * D;
   if constexpr (!FP8) {
-    // same-dtype cache: 16-byte pieces of the staged K row and of the V row
-    const int64_t row_bytes = (int64_t)row * es;
-    uint8_t* kd = p.k_cache + slot * row_bytes;
-    uint8_t* vd = p.v_cache + slot * row_bytes;
-    for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kNormThreads * 16) {
-      *(uint4*)(kd + off) = *(const uint4*)((const uint8_t*)krow + off);
-      *(uint4*)(vd + off) = *(const uint4*)(vsrc + off);
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) {
+        store8_from_f32(p.k_cache, slot * row + (int64_t)head * D + c * 8, DT, kx[g]);
+        store8_from_f32(p.v_cache, slot * row + (int64_t)head * D + c * 8, DT, vx[g]);
+      }
     }
   } else {
-    // quantising cache: per-token amax over all heads, scale = (1/amax) * 448, e4m3fn bytes
-    auto quantise = [&](const void* src_row, uint8_t* dst, float* scale_dst) {
-      float amax = 0.0f;
-      for (int e = threadIdx.x * 8; e < row; e += kNormThreads * 8) {
-        float x[8];
-        load8_as_f32(src_row, e, p.dtype, x);
+    // per-token amax over all heads, scale = (1/amax) * 448, e4m3fn bytes; rows of dead lanes are zero
+    float ka = 0.0f, va = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) amax = nan_keeping_max(amax, fabsf(x[j]));
+    for (int g = 0; g < kMaxKvGroups; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ka = nan_keeping_max(ka, fabsf(kx[g][e]));
+        va = nan_keeping_max(va, fabsf(vx[g][e]));
       }
-      const float s = block_scale(amax, red, wave, lane);
-      if (threadIdx.x == 0) *scale_dst = s;
-      for (int e = threadIdx.x * 8; e < row; e += kNormThreads * 8) {
-        float x[8];
-        load8_as_f32(src_row, e, p.dtype, x);
-        uint32_t w[2];
+    const float ksc = wave_scale(ka), vsc = wave_scale(va);
+    if (lane == 0) {
+      p.k_scale[slot] = ksc;
+      p.v_scale[slot] = vsc;
+    }
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          uint32_t b = 0;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) b |= f32_to_e4m3fn(__fmul_rn(x[4 * j + k], s)) << (8 * k);
-          w[j] = b;
-        }
-        *(uint2*)(dst + e) = make_uint2(w[0], w[1]);
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) {
+        *(uint2*)(p.k_cache + slot * row + (int64_t)head * D + c * 8) = encode8(kx[g], ksc);
+        *(uint2*)(p.v_cache + slot * row + (int64_t)head * D + c * 8) = encode8(vx[g], vsc);
       }
-    };
-    quantise(krow, p.k_cache + slot * row, p.k_scale + slot);
-    quantise(vsrc, p.v_cache + slot * row, p.v_scale + slot);
+    }
   }
 }
 
@@ -229,8 +279,14 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
   if (head_dim != 64 && head_dim != 128)
     return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: head_dim must be 64 or 128");
   const int es = dtype == PA_DTYPE_F32 ? 4 : 2;
-  if (num_kv_heads * head_dim * es > kMaxRow * 2)
-    return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: kv_heads * head_dim too large for the staging row");
+  if (num_kv_heads * head_dim > kMaxKvGroups * 512)
+    return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: kv_heads * head_dim must not exceed 2048");
+  // every row is moved in 16-byte pieces
+  const auto rows16 = [&](const void* base, int64_t stride) { return aligned16(base) && (stride * es) % 16 == 0; };
+  if (!rows16(q, q_token_stride) || !rows16(k, k_token_stride) || !rows16(q_out, q_out_token_stride) ||
+      (k_out && !rows16(k_out, k_out_token_stride)) || !aligned16(q_norm_weight) || !aligned16(k_norm_weight) ||
+      !aligned16(inv_freq))
+    return fail(PA_ERR_BAD_ARG, "pa_qk_norm_rope_store: rows, weights and inv_freq must be 16-byte aligned");
   if (q_token_stride < num_q_heads * head_dim || q_out_token_stride < num_q_heads * head_dim ||
       k_token_stride < num_kv_heads * head_dim || (k_out && k_out_token_stride < num_kv_heads * head_dim))
     return fail(PA_ERR_BAD_ARG, "pa_qk_norm_rope_store: token stride smaller than a row");
@@ -247,8 +303,6 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
       return fail(PA_ERR_BAD_ARG, "pa_qk_norm_rope_store: v rows and caches must be 16-byte aligned");
   }
   if (num_tokens > 0x7fffffff) return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: too many tokens");
-  if (num_q_heads + num_kv_heads > 4 * kNormWaves)
-    return fail(PA_ERR_UNSUPPORTED, "pa_qk_norm_rope_store: more than 32 q + kv heads per token");
 
   NormRopeParams p;
   p.q = q; p.k = k; p.v = v;
@@ -260,18 +314,27 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
   p.k_cache = (uint8_t*)k_cache; p.v_cache = (uint8_t*)v_cache;
   p.k_scale = k_scale; p.v_scale = v_scale;
   p.slot_mapping = slot_mapping; p.total_slots = total_slots;
+  p.num_tokens = num_tokens;
   p.dtype = dtype; p.weight_dtype = weight_dtype;
   p.hq = (int)num_q_heads; p.hkv = (int)num_kv_heads;
   p.eps = eps;
 
-  dim3 grid((unsigned)num_tokens);
+  dim3 grid((unsigned)((num_tokens + kTokensPerGroup - 1) / kTokensPerGroup));
   hipStream_t st = (hipStream_t)stream;
-  if (head_dim == 128) {
-    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, true>), grid, dim3(kNormThreads), 0, st, p);
-    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<128, false>), grid, dim3(kNormThreads), 0, st, p);
-  } else {
-    if (fp8) hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, true>), grid, dim3(kNormThreads), 0, st, p);
-    else hipLaunchKernelGGL((qk_norm_rope_store_kernel<64, false>), grid, dim3(kNormThreads), 0, st, p);
+#define PA_LAUNCH_NORM_ROPE(DIM, F8, DT) \
+  hipLaunchKernelGGL((qk_norm_rope_store_kernel<DIM, F8, DT>), grid, dim3(64 * kTokensPerGroup), 0, st, p)
+#define PA_LAUNCH_NORM_ROPE_DT(DIM, F8)                                  \
+  switch (dtype) {                                                       \
+    case PA_DTYPE_F16: PA_LAUNCH_NORM_ROPE(DIM, F8, PA_DTYPE_F16); break;   \
+    case PA_DTYPE_BF16: PA_LAUNCH_NORM_ROPE(DIM, F8, PA_DTYPE_BF16); break; \
+    default: PA_LAUNCH_NORM_ROPE(DIM, F8, PA_DTYPE_F32); break;             \
   }
+  if (head_dim == 128) {
+    if (fp8) { PA_LAUNCH_NORM_ROPE_DT(128, true) } else { PA_LAUNCH_NORM_ROPE_DT(128, false) }
+  } else {
+    if (fp8) { PA_LAUNCH_NORM_ROPE_DT(64, true) } else { PA_LAUNCH_NORM_ROPE_DT(64, false) }
+  }
+#undef PA_LAUNCH_NORM_ROPE_DT
+#undef PA_LAUNCH_NORM_ROPE
   return check_launch("pa_qk_norm_rope_store");
 }

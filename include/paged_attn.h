@@ -214,7 +214,7 @@ int pa_f32_to_fp8_e4m3(const float* src, void* dst, int64_t n, void* stream);
  *   pa_kv_store (kv_dtype == dtype) or pa_kv_store_fp8 (kv_dtype == PA_DTYPE_FP8_E4M3, per-token
  *   scales to k_scale / v_scale) would write them; slot < 0 or >= total_slots: no cache write.
  *   k_cache == NULL: no cache write at all (v, v_cache, scales, slot_mapping unused).
- * head_dim 64 or 128; Hkv * D * sizeof(dtype) <= 8192; Hq + Hkv <= 32.
+ * head_dim 64 or 128; Hkv * D <= 2048; q, k, v, q_out, k_out rows, the weights and inv_freq 16-byte aligned.
  * Replaces: RMSNorm.forward on q and k (src/distributed/tensor_parallel.py:78-84, used at
  * :453-454), _apply_rotary_emb (:394-419, used at :457-464) and store_kv_cache
  * (src/inference/attention.py:44-183) of one attention layer.
