@@ -177,17 +177,24 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
 
   // ---- query: GC heads x EPL elements per lane, pre-multiplied by scale*log2(e) -------------
   float qf[GC][EPL];
+  // the dtype switch sits outside the loops: inside, it would put a branch and a wait between
+  // loads that are meant to be in flight together
+  auto load_q = [&](auto dt_tag) __attribute__((always_inline)) {
 #pragma unroll
-  for (int h = 0; h < GC; ++h) {
-    const int64_t base = b * p.q_stride + (int64_t)(hq + h) * D;
+    for (int h = 0; h < GC; ++h) {
+      const int64_t base = b * p.q_stride + (int64_t)(hq + h) * D;
 #pragma unroll
-    for (int k = 0; k < EPL; k += 8) {
-      float x[8];
-      load8_as_f32(p.q, base + G::dim_of(k, j), p.q_dtype, x);
+      for (int k = 0; k < EPL; k += 8) {
+        float x[8];
+        load8_as_f32(p.q, base + G::dim_of(k, j), decltype(dt_tag)::value, x);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qf[h][k + e] = x[e] * p.scale_log2e;
+        for (int e = 0; e < 8; ++e) qf[h][k + e] = x[e] * p.scale_log2e;
+      }
     }
-  }
+  };
+  if (p.q_dtype == PA_DTYPE_F16) load_q(std::integral_constant<int, PA_DTYPE_F16>{});
+  else if (p.q_dtype == PA_DTYPE_BF16) load_q(std::integral_constant<int, PA_DTYPE_BF16>{});
+  else load_q(std::integral_constant<int, PA_DTYPE_F32>{});
 
   float m[GC], l[GC], acc[GC][EPL];
 #pragma unroll

@@ -217,13 +217,20 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
   {
     const int tq = min(tok, lq - 1);
     const int64_t base = (int64_t)(q0 + tq) * p.q_stride + (int64_t)qhead * D + 8 * h;
+    // the dtype switch sits outside the loop: inside, it would put a branch and a wait between
+    // loads that are meant to be in flight together
+    auto load_q = [&](auto dt_tag) __attribute__((always_inline)) {
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      float x[8];
-      load8_as_f32(p.q, base + ks * 16, p.q_dtype, x);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        float x[8];
+        load8_as_f32(p.q, base + ks * 16, decltype(dt_tag)::value, x);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qreg[ks][e] = (_Float16)x[e];
-    }
+        for (int e = 0; e < 8; ++e) qreg[ks][e] = (_Float16)x[e];
+      }
+    };
+    if (p.q_dtype == PA_DTYPE_F16) load_q(std::integral_constant<int, PA_DTYPE_F16>{});
+    else if (p.q_dtype == PA_DTYPE_BF16) load_q(std::integral_constant<int, PA_DTYPE_BF16>{});
+    else load_q(std::integral_constant<int, PA_DTYPE_F32>{});
   }
 
   float16_t o[MT];
