@@ -292,7 +292,8 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-seqs", type=int, default=8)
+    ap.add_argument("--cpu-sample-seqs", type=int, default=64,
+                    help="sequences of the batch the CPU baseline decodes (default: all of them)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the auxiliary measurements (KV store, fused q/k kernel, sampler, model step): "
                          "keeps a profiler trace of the run small")
@@ -371,7 +372,7 @@ def main():
             sample_bytes = algorithmic_bytes(n, CTX, HQ, HKV, D, BS, False)
             results["cpu"] = dict(value=sample_bytes / sec / 1e9, unit="GB/s",
                                   cores=torch.get_num_threads(), kind="port",
-                                  sample="oracle decode (per-sequence gather + SDPA) of the first %d of %d "
+                                  sample="oracle decode (per-sequence gather + SDPA) of %d of the %d "
                                          "sequences, ctx %d, FP16 KV, best of 3: %.1f ms; "
                                          "host has %d logical CPUs; max |gpu-cpu| on the sample %.2e"
                                          % (n, B, CTX, sec * 1e3, os.cpu_count(), err),
