@@ -11,6 +11,7 @@ loader module at the repository root.
 from .context import InferenceContext, set_context, get_context, reset_context
 from .kv_cache import Block, BlockPool, BlockTable, KVCacheManager, HAS_FP8, _FP8_DTYPE
 from .prefix_cache import PrefixCache, CachedBlock
+from .radix_cache import RadixAttentionCache, RadixNode
 from .attention import (
     PagedAttention,
     PartitionedPagedAttention,
@@ -29,7 +30,7 @@ from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",

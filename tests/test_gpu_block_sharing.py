@@ -161,3 +161,130 @@ def test_k_samples_share_prompt_blocks_and_decode_like_private_copies(pa, gpu, c
     for s in seqs:
         mgr.free_sequence(s)
     assert pool.num_free_blocks == pool.num_blocks
+
+
+@pytest.mark.parametrize("kind", ["hash-chain", "radix"])
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_requests_reuse_a_cached_prompt_prefix_and_prefill_only_their_tails(pa, gpu, cache, kind):
+    """The engine's prefix path (src/inference/engine.py:582-616) with the reuse made real: a
+    request looks its prompt up, aliases the matched blocks, stores K/V for the unmatched tail
+    only and runs chunked prefill over cached prefix + tail; then everything decodes one step.
+    Checked against the oracle on a private pool holding every request's whole history."""
+    BS, HQ, HKV, D, L = 16, 16, 8, 128, 2
+    pool = pkg.BlockPool(96, BS, num_layers=L, num_kv_heads=HKV, head_dim=D, device=gpu, cache_dtype=cache)
+    mgr = pkg.KVCacheManager(pool, BS)
+    lookup = (pkg.PrefixCache(BS, 64, block_pool=pool) if kind == "hash-chain"
+              else pkg.RadixAttentionCache(BS, 64, block_pool=pool))
+    g = torch.Generator().manual_seed(1044)
+    rnd = lambda *s: torch.randn(*s, generator=g).half()
+    scale = D ** -0.5
+    tol = dict(rtol=1e-2, atol=1e-2) if cache == "fp8" else dict(rtol=1e-3, atol=2e-3)
+
+    system = list(range(1000, 1000 + 5 * BS))                      # 80 tokens, 5 full blocks
+    turn = [7000 + i for i in range(2 * BS + 3)]                   # a second shared stretch, ends mid-block
+    prompts = [
+        system + [2000 + i for i in range(21)],
+        system + [3000 + i for i in range(40)],                    # same system prompt, other question
+        system + turn + [4000 + i for i in range(9)],
+        system + turn + [5000 + i for i in range(30)],             # shares system + 2 blocks of the turn
+        system + [2000 + i for i in range(21)] + [6000, 6001],     # request 0 again, two tokens longer
+    ]
+    expect_matched = [0, 5 * BS, 5 * BS, 7 * BS, 6 * BS]
+
+    def private_pool(rows):
+        nb = sum((r + BS - 1) // BS for r in rows)
+        pk = torch.zeros(nb, BS, HKV, D, dtype=torch.float16)
+        pv = torch.zeros_like(pk)
+        pks = torch.ones(nb, BS) if cache == "fp8" else None
+        pvs = torch.ones(nb, BS) if cache == "fp8" else None
+        if cache == "fp8":
+            pk, pv = pk.to(torch.float8_e4m3fn), pv.to(torch.float8_e4m3fn)
+        return pk, pv, pks, pvs
+
+    hist = {}                   # request -> per layer (k, v) of all its tokens, owned by nobody else
+    owner_of = {}               # prompt prefix (as tuple, block aligned) -> request that computed it
+    for r, tokens in enumerate(prompts):
+        matched, ids = lookup.match_prefix(tokens)
+        assert matched == expect_matched[r] and len(ids) == matched // BS
+        assert mgr.can_allocate(len(tokens), num_shared_blocks=len(ids))
+        before = pool.num_used_blocks
+        table = mgr.allocate_for_sequence(r, len(tokens), shared_block_ids=ids).get_physical_block_ids()
+        assert table[:len(ids)] == ids
+        assert pool.num_used_blocks - before == (len(tokens) + BS - 1) // BS - len(ids)   # only the tail costs blocks
+        tail = len(tokens) - matched
+        slots = torch.tensor([table[i // BS] * BS + i % BS for i in range(matched, len(tokens))], dtype=torch.int32)
+        src = owner_of.get(tuple(tokens[:matched]))
+        hist[r] = []
+        for layer in range(L):
+            k_new, v_new = rnd(tail, HKV, D), rnd(tail, HKV, D)
+            kc, vc, ks, vs = pool.layer_views(layer)
+            pa.store_kv_cache(k_new.to(gpu), v_new.to(gpu), kc, vc, slots.to(gpu), ks, vs, cache_dtype=cache)
+            if matched:
+                k_old, v_old = hist[src][layer]
+                k_new, v_new = torch.cat([k_old[:matched], k_new]), torch.cat([v_old[:matched], v_new])
+            hist[r].append((k_new, v_new))
+
+            # chunked prefill of the tail over the aliased prefix
+            q = rnd(tail, HQ, D)
+            cu_q = torch.tensor([0, tail], dtype=torch.int32)
+            cu_k = torch.tensor([0, len(tokens)], dtype=torch.int32)
+            bt = torch.tensor([table], dtype=torch.int32)
+            got = pa.paged_prefill(q.to(gpu), kc, vc, cu_q.to(gpu), cu_k.to(gpu), tail, scale,
+                                   block_tables=bt.to(gpu), k_scale=ks, v_scale=vs).cpu()
+            pk, pv, pks, pvs = private_pool([len(tokens)])
+            oracle.store_kv_cache(k_new, v_new, pk, pv, torch.arange(len(tokens), dtype=torch.int32), pks, pvs, cache)
+            pbt = torch.arange(pk.shape[0], dtype=torch.int32)[None]
+            want = oracle.prefill_paged(q, pk, pv, pbt, cu_q, cu_k, scale, pks, pvs, cache)
+            torch.testing.assert_close(got.float(), want.float(), **tol)
+        lookup.insert(tokens, table)
+        for n_blocks in range(1, len(tokens) // BS + 1):
+            owner_of.setdefault(tuple(tokens[:n_blocks * BS]), r)
+        if kind == "radix":
+            lookup.release_prefix(tokens, matched // BS)
+        else:
+            for h in lookup.block_hashes(tokens, matched // BS):
+                lookup.release_block(h)
+
+    # the system prompt's blocks: one physical copy, referenced by five requests and the cache
+    tables = [mgr.get_block_table(r) for r in range(len(prompts))]
+    assert all(t[:5] == tables[0][:5] for t in tables)
+    assert all(pool.get_block(b).ref_count == len(prompts) + 1 for b in tables[0][:5])
+    assert tables[3][5:7] == tables[2][5:7] and tables[4][5] == tables[0][5]
+    assert pool.num_used_blocks == len({b for t in tables for b in t})
+
+    # one decode step for all requests; the new token never lands in a shared block
+    seqs = list(range(len(prompts)))
+    slots = []
+    for s in seqs:
+        assert mgr.append_token(s)
+        slots.append(mgr.next_slot(s))
+        assert pool.get_block(slots[-1] // BS).ref_count == 1
+    mgr.apply_copies()
+    lens = [mgr.get_seq_token_count(s) for s in seqs]
+    width = max(len(mgr.get_block_table(s)) for s in seqs)
+    bt = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    for i, s in enumerate(seqs):
+        ids = mgr.get_block_table(s)
+        bt[i, :len(ids)] = torch.tensor(ids, dtype=torch.int32)
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    for layer in range(L):
+        k1, v1, q = rnd(len(seqs), HKV, D), rnd(len(seqs), HKV, D), rnd(len(seqs), HQ, D)
+        kc, vc, ks, vs = pool.layer_views(layer)
+        pa.store_kv_cache(k1.to(gpu), v1.to(gpu), kc, vc, torch.tensor(slots, dtype=torch.int32, device=gpu),
+                          ks, vs, cache_dtype=cache)
+        got = pa.paged_decode(q.to(gpu), kc, vc, bt.to(gpu), ctx.to(gpu), scale, ks, vs).cpu()
+        pk, pv, pks, pvs = private_pool([width * BS] * len(seqs))
+        pbt = torch.arange(len(seqs) * width, dtype=torch.int32).view(len(seqs), width)
+        for i, s in enumerate(seqs):
+            k = torch.cat([hist[s][layer][0], k1[i:i + 1]])
+            v = torch.cat([hist[s][layer][1], v1[i:i + 1]])
+            sl = torch.arange(k.shape[0], dtype=torch.int32) + i * width * BS
+            oracle.store_kv_cache(k, v, pk, pv, sl, pks, pvs, cache)
+        want = oracle.decode(q, pk, pv, pbt, ctx, scale, pks, pvs, cache)
+        torch.testing.assert_close(got.float(), want.float(), **tol)
+
+    for s in seqs:
+        mgr.free_sequence(s)
+    assert pool.num_used_blocks == lookup.size          # what is left belongs to the cache
+    lookup.invalidate_all()
+    assert pool.num_free_blocks == pool.num_blocks
