@@ -12,12 +12,14 @@ from .context import InferenceContext, set_context, get_context, reset_context
 from .kv_cache import Block, BlockPool, BlockTable, KVCacheManager, HAS_FP8, _FP8_DTYPE
 from .prefix_cache import PrefixCache, CachedBlock
 from .radix_cache import RadixAttentionCache, RadixNode
+from .cuda_graph import CUDAGraphRunner
 from .attention import (
     PagedAttention,
     PartitionedPagedAttention,
     store_kv_cache,
     qk_norm_rope_store,
     sample_tokens,
+    slot_mapping,
     paged_decode,
     paged_prefill,
     choose_partition,
@@ -30,7 +32,7 @@ from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "slot_mapping", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",

@@ -50,6 +50,7 @@ SIGNATURES = {
                                      _i64, _i64, _i64, _i64, _ptr]),
     "pa_sample": (_int, [_ptr, _int, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr]),
     "pa_copy_blocks": (_int, [_ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
+    "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_set_decode_waves": (_int, [_int]),
     "pa_get_decode_waves": (_int, []),
     "pa_set_decode_pair_heads": (_int, [_int]),

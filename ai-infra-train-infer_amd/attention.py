@@ -257,6 +257,42 @@ def sample_tokens(logits, temperature=0.7, top_p=0.9, uniforms=None, generator=N
     return out
 
 
+def slot_mapping(positions, block_tables, block_size, num_blocks, cu_seqlens_q=None, out=None):
+    """int32 [tokens] of physical cache slots, computed on the GPU without a host round trip:
+    block_tables[row][position // block_size] * block_size + position % block_size.  Without
+    cu_seqlens_q token i uses table row i (one new token per sequence, the loop at
+    src/inference/model_runner.py:670-682); with it, row = the sequence whose chunk holds the
+    token (model_runner.py:493-511).  Tokens whose position falls outside their table, or on a
+    block id outside the pool (padding -1 included), get -1 and are skipped by the KV writers."""
+    _require_gpu(positions, "slot_mapping")
+    _require_gpu(block_tables, "slot_mapping")
+    if block_tables.dim() != 2:
+        raise RuntimeError("slot_mapping: block_tables must be [rows, max_blocks]")
+    lib = _native.load()
+    positions = positions.reshape(-1)
+    if positions.dtype != torch.int64:
+        positions = positions.to(torch.int64)
+    positions = positions.contiguous()
+    tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+    if tables.stride(1) != 1:
+        tables = tables.contiguous()
+    n = positions.numel()
+    if out is None:
+        out = torch.empty(n, dtype=torch.int32, device=positions.device)
+    elif out.dtype != torch.int32 or out.numel() != n or not out.is_contiguous():
+        raise RuntimeError("slot_mapping: out must be contiguous int32 [tokens]")
+    cu = None
+    if cu_seqlens_q is not None:
+        cu = _int32(cu_seqlens_q, "slot_mapping")
+        if cu.numel() != tables.size(0) + 1:
+            raise RuntimeError("slot_mapping: cu_seqlens_q must have rows + 1 entries")
+    rc = lib.pa_slot_mapping(positions.data_ptr(), cu.data_ptr() if cu is not None else None, tables.data_ptr(),
+                             tables.stride(0), out.data_ptr(), n, tables.size(0), tables.size(1), int(block_size),
+                             int(num_blocks), _stream_ptr(positions.device))
+    _native.check(rc, "pa_slot_mapping")
+    return out
+
+
 def _workspace(device, nbytes):
     """Per (device, stream) scratch for the partition partials; grows, never shrinks."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)

@@ -1,0 +1,70 @@
+// Physical cache slots of tokens, computed on the device (gfx950).
+//
+// The reference's batched decode derives the slot of every sequence's new token on the host,
+// reading position and block id back from the GPU one element at a time
+// (src/inference/model_runner.py:670-680: two .item() synchronisations per sequence), and its
+// prefill builds the same list in Python loops (model_runner.py:493-511).  Both are
+//     slot(token) = block_table[row][position / block_size] * block_size + position % block_size
+// over tensors that already sit in HBM, so one small launch does it without leaving the stream:
+// one thread per token; the token's table row is its own index (decode) or is found by bisection
+// of cu_seqlens_q (prefill chunks).  A position that is negative or beyond the table, and a
+// block id outside the pool, give slot -1, which the KV writers skip.
+#include "pa_common.hpp"
+#include "pa_host.hpp"
+
+namespace pa {
+
+__global__ __launch_bounds__(256) void slot_mapping_kernel(const int64_t* __restrict__ positions,
+                                                           const int32_t* __restrict__ cu_seqlens_q,
+                                                           const int32_t* __restrict__ block_tables,
+                                                           int64_t bt_stride, int32_t* __restrict__ slots,
+                                                           int64_t num_tokens, int num_rows, int table_width,
+                                                           int block_size, int num_blocks) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= num_tokens) return;
+  int row;
+  if (cu_seqlens_q) {
+    // last row whose first token is <= t; rows without tokens are passed over
+    int lo = 0, hi = num_rows;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if ((int64_t)cu_seqlens_q[mid] <= t) lo = mid; else hi = mid;
+    }
+    row = lo;
+    if (t >= (int64_t)cu_seqlens_q[num_rows]) { slots[t] = -1; return; }
+  } else {
+    row = (int)t;
+  }
+  const int64_t pos = positions[t];
+  int32_t slot = -1;
+  if (pos >= 0 && pos / block_size < table_width) {
+    const int32_t block = block_tables[(int64_t)row * bt_stride + pos / block_size];
+    if (block >= 0 && block < num_blocks) slot = block * block_size + (int32_t)(pos % block_size);
+  }
+  slots[t] = slot;
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+extern "C" int pa_slot_mapping(const int64_t* positions, const int32_t* cu_seqlens_q, const int32_t* block_tables,
+                               int64_t bt_stride, int32_t* slots, int64_t num_tokens, int64_t num_rows,
+                               int64_t table_width, int64_t block_size, int64_t num_blocks, void* stream) {
+  if (num_tokens < 0 || num_rows < 0 || table_width < 0 || block_size <= 0 || num_blocks <= 0)
+    return fail(PA_ERR_BAD_ARG, "pa_slot_mapping: negative or zero size");
+  if (num_tokens == 0) return PA_OK;
+  if (!positions || !block_tables || !slots) return fail(PA_ERR_BAD_ARG, "pa_slot_mapping: null pointer");
+  if (num_rows == 0) return fail(PA_ERR_BAD_ARG, "pa_slot_mapping: tokens but no table rows");
+  if (!cu_seqlens_q && num_tokens != num_rows)
+    return fail(PA_ERR_BAD_ARG, "pa_slot_mapping: without cu_seqlens_q every table row has exactly one token");
+  if (bt_stride < table_width) return fail(PA_ERR_BAD_ARG, "pa_slot_mapping: table stride smaller than its width");
+  if (num_rows > INT32_MAX || table_width > INT32_MAX || num_blocks * block_size > INT32_MAX)
+    return fail(PA_ERR_UNSUPPORTED, "pa_slot_mapping: slots must fit int32");
+  const int64_t wgs = (num_tokens + 255) / 256;
+  if (wgs > INT32_MAX) return fail(PA_ERR_UNSUPPORTED, "pa_slot_mapping: too many tokens for one launch");
+  hipLaunchKernelGGL(slot_mapping_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, positions,
+                     cu_seqlens_q, block_tables, bt_stride, slots, num_tokens, (int)num_rows, (int)table_width,
+                     (int)block_size, (int)num_blocks);
+  return check_launch("pa_slot_mapping");
+}

@@ -3,7 +3,8 @@
 Mirrors the part of the reference's ModelRunner that feeds the attention layers
 (src/inference/model_runner.py): `bind_kv_cache` / `_bind_kv_cache_to_model` (:78-116),
 `prepare_prefill` (:464-540), `prepare_decode` (:542-588), `_prepare_block_tables` (:814-828),
-`run` (:128-165) and the decode graph capture / replay (:710-810).  Same sequence dictionaries in,
+`run` (:128-165), `run_batch_decode` (:639-708), `sample` (:590-634) and the decode graph capture /
+replay (:710-810).  Same sequence dictionaries in,
 same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_tables` padded with
 -1).  What differs is how the metadata reaches the GPU:
 
@@ -12,10 +13,11 @@ same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_t
     torch.tensor(...) per field; here every field is filled in one pinned host staging buffer
     with numpy row copies and shipped with a single asynchronous copy per step;
   * graph replay copies into static device buffers and pads with slot -1 / context 0, exactly as
-    the reference does, but capture needs no host synchronisation inside the model.
+    the reference does, but capture needs no host synchronisation inside the model;
+  * `run_batch_decode` gets its slot mapping from a kernel instead of two `.item()` reads per
+    sequence, so a decode step driven by device-resident tables never waits for the GPU.
 
-Sampling, HF-model KV gathering and mock logits are host policy outside this path and are not
-rebuilt.
+HF-model KV gathering and mock logits are outside this path and are not rebuilt.
 """
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
@@ -188,6 +190,22 @@ class ModelRunner:
             logits = self.model(input_ids, positions=positions)
         reset_context()
         return logits
+
+    @torch.inference_mode()
+    def run_batch_decode(self, input_ids, positions, block_tables, context_lens):
+        """One decode step for a batch whose metadata is already on the GPU: input_ids [batch] or
+        [batch, 1], positions [batch] (of the token being written), block_tables [batch, max_blocks]
+        int32, context_lens [batch] int32 (counting that token) -> logits [batch, vocab]
+        (src/inference/model_runner.py:639-708)."""
+        if self.model is None:
+            raise RuntimeError("ModelRunner.run_batch_decode: no model bound")
+        from .attention import slot_mapping
+        if input_ids.dim() == 2:
+            input_ids = input_ids.squeeze(1)
+        num_blocks = self._kv_cache.shape[2] if self._kv_cache is not None else 2 ** 31 // self.block_size - 1
+        slots = slot_mapping(positions, block_tables, self.block_size, num_blocks)
+        set_context(is_prefill=False, slot_mapping=slots, context_lens=context_lens, block_tables=block_tables)
+        return self.run(input_ids, positions, is_prefill=False)
 
     # ---------------------------------------------------------------- sampling
 

@@ -244,6 +244,22 @@ int pa_sample(const void* logits, int dtype, int64_t row_stride, int64_t batch, 
               float temperature, float top_p, const float* uniforms, int64_t* out, void* stream);
 
 /*
+ * slots[t] = block_tables[row(t)][positions[t] / block_size] * block_size + positions[t] % block_size
+ * for num_tokens tokens, all on the device.  cu_seqlens_q == NULL: token t belongs to table row t
+ * (one new token per sequence, num_tokens == num_rows).  Otherwise cu_seqlens_q is int32
+ * [num_rows + 1] and row(t) is the sequence whose chunk [cu[r], cu[r+1]) holds t; tokens at or
+ * past cu[num_rows] get -1.  positions is int64 (the reference's `positions` tensors are
+ * torch.long).  A negative position, a position past table_width blocks, or a block id outside
+ * [0, num_blocks) gives -1, which pa_kv_store / pa_kv_store_fp8 / pa_qk_norm_rope_store skip.
+ * Replaces: the per-sequence host loop of ModelRunner.run_batch_decode
+ * (src/inference/model_runner.py:670-682, two .item() reads per sequence) and the slot loops of
+ * prepare_prefill (model_runner.py:493-511).
+ */
+int pa_slot_mapping(const int64_t* positions, const int32_t* cu_seqlens_q, const int32_t* block_tables,
+                    int64_t bt_stride, int32_t* slots, int64_t num_tokens, int64_t num_rows,
+                    int64_t table_width, int64_t block_size, int64_t num_blocks, void* stream);
+
+/*
  * Copy whole cache blocks inside one pool tensor laid out [num_planes][num_blocks][block_bytes]
  * (planes plane_stride_bytes apart): for every plane and every pair i, block pairs[2i+1] := block
  * pairs[2i].  The K/V tensor of a BlockPool is one such tensor with 2 x layers planes, each fp8

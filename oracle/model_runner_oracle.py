@@ -4,6 +4,7 @@ metadata (TEST INFRASTRUCTURE ONLY; plain Python loops, lists out):
   prefill_metadata   src/inference/model_runner.py:464-540
   decode_metadata    src/inference/model_runner.py:542-588
   block_tables       src/inference/model_runner.py:814-828
+  batch_decode_slots src/inference/model_runner.py:670-682
 
 Pinned by the closed form "slot of position p = block_table[p // BS] * BS + p % BS" in
 tests/test_model_runner_host.py.
@@ -70,3 +71,18 @@ def decode_metadata(sequences, block_size):
         context_lens.append(len(seq["token_ids"]))
     return dict(input_ids=input_ids, positions=positions, slot_mapping=slot_mapping,
                 context_lens=context_lens, block_tables=block_tables(sequences))
+
+
+def batch_decode_slots(positions, block_tables, block_size):
+    """src/inference/model_runner.py:670-682: the slot of each sequence's new token, read from
+    its own table row.  (The reference indexes without checks; rows whose position falls
+    outside the table, or on a padding id, are reported as None here.)"""
+    slots = []
+    for i, token_pos in enumerate(positions):
+        block_idx = token_pos // block_size
+        offset = token_pos % block_size
+        if token_pos < 0 or block_idx >= len(block_tables[i]) or block_tables[i][block_idx] < 0:
+            slots.append(None)
+            continue
+        slots.append(block_tables[i][block_idx] * block_size + offset)
+    return slots

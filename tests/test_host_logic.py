@@ -70,3 +70,20 @@ def test_block_pool_layout(pa):
     model = torch.nn.Sequential(pa.PagedAttention(16, 8, 128), pa.PartitionedPagedAttention(16, 8, 128))
     assert pool.bind_to_model(model) == 2
     assert model[1].k_cache.data_ptr() == k.data_ptr() and model[1].cache_dtype == "fp8"
+
+
+def test_graph_runner_host_side_without_a_gpu():
+    """Size ladder and fallbacks of CUDAGraphRunner (src/inference/cuda_graph.py:41-56, 197-233)."""
+    import ai_infra_train_infer_amd as pkg
+    r = pkg.CUDAGraphRunner(max_batch_size=20)
+    assert r.supported_batch_sizes == [1, 2, 4, 8, 16]
+    assert [r._get_padded_batch_size(b) for b in (1, 3, 8, 9, 16, 17)] == [1, 4, 8, 16, 16, None]
+    assert pkg.CUDAGraphRunner(max_batch_size=0).supported_batch_sizes == [1]
+    assert pkg.CUDAGraphRunner(supported_batch_sizes=[8, 2]).supported_batch_sizes == [2, 8]
+    if not torch.cuda.is_available():
+        r.capture(lambda ids, pos: ids, 4, (4,))                      # no GPU: quietly does nothing
+    assert not r.is_captured(4) and r.replay(4, torch.zeros(4, dtype=torch.long)) is None
+    st = r.get_stats()
+    assert st == {"captured_sizes": [], "total_captures": 0, "total_replays": 0, "graph_pool_active": False,
+                  "supported_batch_sizes": [1, 2, 4, 8, 16]}
+    r.invalidate()
