@@ -257,6 +257,75 @@ def sample_tokens(logits, temperature=0.7, top_p=0.9, uniforms=None, generator=N
     return out
 
 
+def _rows2d(t, what):
+    """[rows, width] view whose rows are 16-byte aligned and unit-stride inside; (tensor, row stride)."""
+    if t.dim() != 2:
+        raise RuntimeError("%s: expected a 2-D tensor, got %s" % (what, tuple(t.shape)))
+    es = t.element_size()
+    if t.stride(1) != 1 or (t.stride(0) * es) % 16 != 0 or t.data_ptr() % 16 != 0:
+        t = t.contiguous()
+    return t, (t.stride(0) if t.shape[0] > 1 else t.shape[1])
+
+
+def add_rms_norm(x, weight, eps=1e-6, delta=None, inplace_sum=True):
+    """RMSNorm of the residual stream, fused with the residual add that precedes it
+    (src/distributed/tensor_parallel.py:78-84 and :640-651).  x [rows, hidden]; with delta
+    [rows, hidden] returns (x + delta, norm(x + delta)) - the sum is written into x when
+    inplace_sum - and without it (x, norm(x)).  Same roundings as the separate ops."""
+    _require_gpu(x, "add_rms_norm")
+    lib = _native.load()
+    shape = x.shape
+    x2, xs = _rows2d(x.reshape(-1, shape[-1]), "add_rms_norm")
+    rows, hidden = x2.shape
+    code = _code(x2.dtype, "add_rms_norm")
+    normed = torch.empty((rows, hidden), dtype=x2.dtype, device=x2.device)
+    if weight.numel() != hidden or not weight.is_contiguous():
+        raise RuntimeError("add_rms_norm: weight must be contiguous [hidden]")
+    d2 = ds = None
+    total = x2
+    if delta is not None:
+        if delta.shape != shape or delta.dtype != x.dtype:
+            raise RuntimeError("add_rms_norm: delta must match x in shape and dtype")
+        d2, ds = _rows2d(delta.reshape(-1, hidden), "add_rms_norm")
+        total = x2 if inplace_sum else torch.empty((rows, hidden), dtype=x2.dtype, device=x2.device)
+    rc = lib.pa_add_rms_norm(x2.data_ptr(), xs, d2.data_ptr() if d2 is not None else None, ds or 0,
+                             weight.data_ptr(), _code(weight.dtype, "add_rms_norm"), float(eps),
+                             total.data_ptr() if d2 is not None else None,
+                             (total.stride(0) if rows > 1 else hidden) if d2 is not None else 0,
+                             normed.data_ptr(), hidden, code, rows, hidden, _stream_ptr(x2.device))
+    _native.check(rc, "pa_add_rms_norm")
+    return total.view(shape), normed.view(shape)
+
+
+def silu_mul(gate, up=None):
+    """silu(gate) * up of a SwiGLU MLP (src/distributed/tensor_parallel.py:295-299).  With one
+    argument [rows, 2 * width] it is the packed gate|up projection output."""
+    _require_gpu(gate, "silu_mul")
+    lib = _native.load()
+    if up is None:
+        if gate.shape[-1] % 2:
+            raise RuntimeError("silu_mul: packed gate|up needs an even width")
+        width = gate.shape[-1] // 2
+        packed, stride = _rows2d(gate.reshape(-1, 2 * width), "silu_mul")
+        if (width * packed.element_size()) % 16 != 0:
+            raise RuntimeError("silu_mul: width must be a multiple of 16 bytes")
+        g, u, gs, us = packed, packed[:, width:], stride, stride
+        lead = gate.shape[:-1]
+    else:
+        if up.shape != gate.shape or up.dtype != gate.dtype:
+            raise RuntimeError("silu_mul: gate and up must match in shape and dtype")
+        width = gate.shape[-1]
+        g, gs = _rows2d(gate.reshape(-1, width), "silu_mul")
+        u, us = _rows2d(up.reshape(-1, width), "silu_mul")
+        lead = gate.shape[:-1]
+    rows = g.shape[0]
+    out = torch.empty((rows, width), dtype=g.dtype, device=g.device)
+    rc = lib.pa_silu_mul(g.data_ptr(), gs, u.data_ptr(), us, out.data_ptr(), width, _code(g.dtype, "silu_mul"),
+                         rows, width, _stream_ptr(g.device))
+    _native.check(rc, "pa_silu_mul")
+    return out.view(*lead, width)
+
+
 def slot_mapping(positions, block_tables, block_size, num_blocks, cu_seqlens_q=None, out=None):
     """int32 [tokens] of physical cache slots, computed on the GPU without a host round trip:
     block_tables[row][position // block_size] * block_size + position % block_size.  Without

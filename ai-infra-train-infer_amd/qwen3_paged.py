@@ -6,10 +6,13 @@ the module a model runner binds caches to (model_runner.py:102-116) and calls as
 `model(input_ids, positions=positions)` (model_runner.py:162).  Block structure follows the
 reference's Qwen3 definition (src/distributed/tensor_parallel.py:307-543): RMSNorm -> q/k/v
 projections -> per-head q/k RMSNorm -> RoPE (half rotation, theta 1e6) -> attention -> o_proj,
-then RMSNorm -> SwiGLU MLP.  GEMMs and the layer norms are plain torch-ROCm ops; the per-head
-q/k norm, the rotation and the KV write are one HIP kernel (`fused_qk`, on by default; off =
-the same steps as separate torch ops), attention another.  Nothing in forward() synchronises with the host, so a
-decode step can be captured in a HIP graph.
+then RMSNorm -> SwiGLU MLP.  GEMMs are torch-ROCm library calls.  Between them a block runs
+five HIP kernels: residual add + RMSNorm, per-head q/k norm + rotation + KV write (`fused_qk`),
+attention, residual add + RMSNorm again, and silu(gate) * up (`fused_elementwise`); both flags are
+on by default, off = the same steps as separate torch ops.  The residual add of a block's MLP
+output is carried into the next block's first norm (and the last one into the final norm), so
+no add is a launch of its own.  Nothing in forward() synchronises with the host, so a decode
+step can be captured in a HIP graph.
 """
 from dataclasses import dataclass
 
@@ -17,7 +20,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .attention import PagedAttention, PartitionedPagedAttention
+from .attention import PagedAttention, PartitionedPagedAttention, add_rms_norm, silu_mul
 from .context import get_context
 
 
@@ -36,6 +39,7 @@ class Qwen3PagedConfig:
     cache_dtype: str = "fp16"
     partition_size: int = 0        # > 0: use PartitionedPagedAttention with this size
     fused_qk: bool = True          # q/k norm + RoPE + cache write as one kernel
+    fused_elementwise: bool = True # residual add + RMSNorm, and silu * up, as one kernel each
 
 
 class RMSNorm(nn.Module):
@@ -76,11 +80,20 @@ class Qwen3PagedLayer(nn.Module):
         self.gate_up_proj = nn.Linear(cfg.hidden_size, 2 * cfg.intermediate_size, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
 
-    def forward(self, x, cos, sin, positions=None, inv_freq=None):
+    def forward(self, x, cos, sin, positions=None, inv_freq=None, delta=None):
+        """x: residual stream [T, hidden]; delta: the previous block's MLP output, not yet added
+        (fused_elementwise only).  Returns (x, delta) for the next block."""
         cfg = self.cfg
         t = x.shape[0]
         q_dim, kv_dim = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
-        qkv = self.qkv_proj(self.input_layernorm(x))
+        fused_ew = cfg.fused_elementwise and x.is_cuda
+        if fused_ew:
+            x, normed = add_rms_norm(x, self.input_layernorm.weight, cfg.rms_norm_eps, delta)
+        else:
+            if delta is not None:
+                x = x + delta
+            normed = self.input_layernorm(x)
+        qkv = self.qkv_proj(normed)
         q = qkv[:, :q_dim].view(t, cfg.num_heads, cfg.head_dim)
         k = qkv[:, q_dim:q_dim + kv_dim].view(t, cfg.num_kv_heads, cfg.head_dim)
         v = qkv[:, q_dim + kv_dim:].view(t, cfg.num_kv_heads, cfg.head_dim)
@@ -91,10 +104,14 @@ class Qwen3PagedLayer(nn.Module):
             q = apply_rope(self.q_norm(q), cos, sin)
             k = apply_rope(self.k_norm(k), cos, sin)
             a = self.attn(q, k, v)                  # writes k, v into the paged cache, then attends
-        x = x + self.o_proj(a.reshape(t, q_dim))
+        o = self.o_proj(a.reshape(t, q_dim))
+        if fused_ew:
+            x, normed = add_rms_norm(x, self.post_attention_layernorm.weight, cfg.rms_norm_eps, o)
+            return x, self.down_proj(silu_mul(self.gate_up_proj(normed)))
+        x = x + o
         gu = self.gate_up_proj(self.post_attention_layernorm(x))
         gate, up = gu[:, :cfg.intermediate_size], gu[:, cfg.intermediate_size:]
-        return x + self.down_proj(F.silu(gate) * up)
+        return x + self.down_proj(F.silu(gate) * up), None
 
 
 class Qwen3PagedModel(nn.Module):
@@ -125,9 +142,16 @@ class Qwen3PagedModel(nn.Module):
         x = self.embed_tokens(input_ids)
         # a model cast with .half() carries its frequency table in 16 bits; both paths use those values
         inv_freq = self.inv_freq.float()
+        delta = None
         for layer in self.layers:
-            x = layer(x, cos, sin, positions, inv_freq)
+            x, delta = layer(x, cos, sin, positions, inv_freq, delta)
         ctx = get_context()
         if ctx.is_prefill and ctx.cu_seqlens_q is not None:
-            x = x[(ctx.cu_seqlens_q[1:] - 1).long()]
-        return self.lm_head(self.norm(x))
+            last = (ctx.cu_seqlens_q[1:] - 1).long()
+            x = x[last]
+            delta = delta[last] if delta is not None else None
+        if self.cfg.fused_elementwise and x.is_cuda:
+            x = add_rms_norm(x, self.norm.weight, self.cfg.rms_norm_eps, delta)[1]
+        else:
+            x = self.norm(x if delta is None else x + delta)
+        return self.lm_head(x)

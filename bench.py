@@ -97,6 +97,20 @@ def time_steps(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps, (t1 - t0) * 1e3 / steps
 
 
+def time_in_graph(torch, fn, steps, warmup, reps=16):
+    """ms per call of `fn` with launch overhead taken out on both sides of a comparison: `reps`
+    calls are recorded into one HIP graph, and the graph is replayed `steps` times."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(reps):
+            fn()
+    ms, _ = time_steps(torch, graph.replay, steps, warmup)
+    return ms / reps
+
+
 def cpu_baseline(torch, w, scale, sample_seqs, bs, repeats=3):
     """The oracle's decode (per-sequence gather + SDPA on the host) over the first
     `sample_seqs` sequences of the workload, compacted into a small pool."""
@@ -214,6 +228,36 @@ def fused_qk_times(pa, torch, dev, steps, warmup):
             rec["algorithmic_bytes"] = alg
             rec["gbps"] = round(alg / ms_f / 1e6, 1)
         out["tokens_%d" % n] = rec
+    return out
+
+
+def block_elementwise_times(pa, torch, dev, steps, warmup):
+    """Residual add + RMSNorm, and silu(gate) * up, of one decoder block at the Qwen3-0.6B shape
+    (hidden 1024, intermediate 3072): the fused kernels beside the same steps as torch ops, for one
+    decode step (64 rows) and one prefill chunk (4096 rows).  Microseconds per call inside a
+    replayed HIP graph (how a decode step runs them); for 4096 rows also the achieved bandwidth over the algorithmic bytes (each input read once, each output written once)."""
+    from ai_infra_train_infer_amd.qwen3_paged import RMSNorm
+    import torch.nn.functional as F
+    H, I = 1024, 3072
+    g = torch.Generator(device=dev).manual_seed(10)
+    norm = RMSNorm(H, 1e-6).to(dev).half()
+    out = {}
+    for n in (64, 4096):
+        x = torch.randn(n, H, generator=g, device=dev, dtype=torch.float32).half()
+        d = torch.randn(n, H, generator=g, device=dev, dtype=torch.float32).half()
+        gu = torch.randn(n, 2 * I, generator=g, device=dev, dtype=torch.float32).half()
+        with torch.inference_mode():
+            ms_nf = time_in_graph(torch, lambda: pa.add_rms_norm(x, norm.weight, 1e-6, delta=d, inplace_sum=False),
+                                  steps, warmup)
+            ms_ns = time_in_graph(torch, lambda: norm(x + d), steps, warmup)
+            ms_sf = time_in_graph(torch, lambda: pa.silu_mul(gu), steps, warmup)
+            ms_ss = time_in_graph(torch, lambda: F.silu(gu[:, :I]) * gu[:, I:], steps, warmup)
+        rec = {"add_rms_norm_us": round(ms_nf * 1e3, 2), "add_rms_norm_torch_ops_us": round(ms_ns * 1e3, 2),
+               "silu_mul_us": round(ms_sf * 1e3, 2), "silu_mul_torch_ops_us": round(ms_ss * 1e3, 2)}
+        if n == 4096:
+            rec["add_rms_norm_gbps"] = round(n * H * 2 * 4 / ms_nf / 1e6, 1)
+            rec["silu_mul_gbps"] = round(n * I * 2 * 3 / ms_sf / 1e6, 1)
+        out["rows_%d" % n] = rec
     return out
 
 
@@ -428,6 +472,7 @@ def main():
     if not args.no_extras:
         line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
+        line["block_elementwise"] = block_elementwise_times(pa, torch, dev, args.steps, args.warmup)
         line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
         line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
     if "cpu" in results:

@@ -244,6 +244,30 @@ int pa_sample(const void* logits, int dtype, int64_t row_stride, int64_t batch, 
               float temperature, float top_p, const float* uniforms, int64_t* out, void* stream);
 
 /*
+ * One decoder block's residual add fused with the RMSNorm that follows it, one row per token:
+ *     s = x + delta            rounded to `dtype` (skipped when delta == NULL: s = x)
+ *     normed = weight * (s * rsqrt(mean(s^2) + eps))      fp32, rounded once to `dtype`
+ * sum_out (optional, needs delta; may alias x or delta) receives s, the residual stream the next
+ * block adds to.  Strides are row strides in elements; rows, weight and bases 16-byte aligned;
+ * hidden a multiple of 8, at most 8192; weight may be f16, bf16 or f32.
+ * Replaces: RMSNorm.forward (src/distributed/tensor_parallel.py:78-84) and the residual adds of
+ * the block (tensor_parallel.py:640-651), seven plus one torch launches.
+ */
+int pa_add_rms_norm(const void* x, int64_t x_stride, const void* delta, int64_t delta_stride,
+                    const void* weight, int weight_dtype, float eps, void* sum_out, int64_t sum_stride,
+                    void* normed_out, int64_t normed_stride, int dtype, int64_t rows, int64_t hidden,
+                    void* stream);
+
+/*
+ * out = silu(gate) * up, element-wise over [rows, width]; silu is rounded to `dtype` before the
+ * product, as F.silu(gate) * up does.  gate and up may be the two halves of one packed
+ * projection output (pass the same row stride).  width a multiple of 8, rows 16-byte aligned.
+ * Replaces: the activation of the SwiGLU MLP (src/distributed/tensor_parallel.py:295-299).
+ */
+int pa_silu_mul(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
+                int64_t out_stride, int dtype, int64_t rows, int64_t width, void* stream);
+
+/*
  * slots[t] = block_tables[row(t)][positions[t] / block_size] * block_size + positions[t] % block_size
  * for num_tokens tokens, all on the device.  cu_seqlens_q == NULL: token t belongs to table row t
  * (one new token per sequence, num_tokens == num_rows).  Otherwise cu_seqlens_q is int32

@@ -9,6 +9,8 @@ do, as the checker.  It follows the reference's module code:
   apply_rotary_emb    src/distributed/tensor_parallel.py:397-419  cos / sin of outer(pos, inv_freq) repeated over both
                                                                   halves; x * cos + cat(-x2, x1) * sin
   qk_norm_rope        src/distributed/tensor_parallel.py:453-464  norm of q and k, then rotation of both
+  add_rms_norm        src/distributed/tensor_parallel.py:640-651  residual + x in the activation dtype, then rms_norm of it
+  swiglu              src/distributed/tensor_parallel.py:295-299  F.silu(gate) * up
 
 The reference's rotation multiplies a 16-bit activation by fp32 cos / sin and therefore returns
 fp32; the block that consumes it casts back to the activation dtype before attention
@@ -22,6 +24,10 @@ Pinning (tests/test_oracle_qwen3_block.py), none of which retypes a formula:
     on m - n only (the property the embedding exists for); pair i at position p has turned by
     exactly p * theta^(-2i/D) radians (checked with atan2 in fp64).
   * qk_norm_rope: equals the two steps applied one after the other.
+  * add_rms_norm: the sum is the correctly rounded sum (checked in fp64); the normed output is
+    rms_norm of that sum.
+  * swiglu: silu(0) = 0, silu(x) -> x for large x and -> 0 for large -x, silu(x) - silu(-x) = x
+    (all in fp64 to rounding), and against x * sigmoid(x) evaluated in fp64.
 """
 import torch
 
@@ -56,3 +62,15 @@ def qk_norm_rope(q, k, q_weight, k_weight, eps, positions, inv_f):
     q = apply_rotary_emb(rms_norm(q, q_weight, eps), positions, inv_f)
     k = apply_rotary_emb(rms_norm(k, k_weight, eps), positions, inv_f)
     return q, k
+
+
+def add_rms_norm(x, delta, weight, eps=1e-6):
+    """(residual + x, norm of it): the block's add is done in the activation dtype, the norm
+    sees the rounded sum."""
+    total = x + delta
+    return total, rms_norm(total, weight, eps)
+
+
+def swiglu(gate, up):
+    import torch.nn.functional as F
+    return F.silu(gate) * up

@@ -58,3 +58,28 @@ def test_qk_norm_rope_is_the_composition():
     qo, ko = ob.qk_norm_rope(q, k, qw, kw, 1e-6, pos, f)
     assert torch.equal(qo, ob.apply_rotary_emb(ob.rms_norm(q, qw, 1e-6), pos, f))
     assert torch.equal(ko, ob.apply_rotary_emb(ob.rms_norm(k, kw, 1e-6), pos, f))
+
+
+def test_add_rms_norm_sum_is_correctly_rounded_and_feeds_the_norm():
+    g = torch.Generator().manual_seed(21)
+    for dt in (torch.float16, torch.bfloat16):
+        x = (torch.randn(7, 256, generator=g) * 3).to(dt)
+        d = torch.randn(7, 256, generator=g).to(dt)
+        w = (torch.rand(256, generator=g) + 0.5).to(dt)
+        total, normed = ob.add_rms_norm(x, d, w, 1e-6)
+        assert torch.equal(total, (x.double() + d.double()).to(dt))       # one rounding of the exact sum
+        assert torch.equal(normed, ob.rms_norm(total, w, 1e-6))
+
+
+def test_swiglu_closed_forms():
+    x = torch.tensor([0.0, 30.0, -30.0, 1.5, -1.5, 0.25, -4.0], dtype=torch.float64)
+    one = torch.ones_like(x)
+    s = ob.swiglu(x, one)
+    assert s[0] == 0 and abs(s[1] - 30.0) < 1e-10 and abs(s[2]) < 1e-10
+    torch.testing.assert_close(ob.swiglu(x, one) - ob.swiglu(-x, one), x, rtol=0, atol=1e-12)
+    torch.testing.assert_close(s, x * torch.sigmoid(x), rtol=1e-12, atol=1e-12)
+    g = torch.Generator().manual_seed(22)
+    gate, up = torch.randn(5, 64, generator=g).half(), torch.randn(5, 64, generator=g).half()
+    want = ((gate.double() * torch.sigmoid(gate.double())).half().double() * up.double()).half()
+    got = ob.swiglu(gate, up)
+    assert (got.float() - want.float()).abs().max() <= 2 ** -10 * want.float().abs().max()
