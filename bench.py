@@ -437,13 +437,14 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate over f16 KV (fp8-e4m3 KV reported beside it)",
+        "dtype": "f32",
         "data": "synthetic N(0,1), seeded, random-permutation block tables",
         "config": {
             "workload": "BASELINE configs[1] shape: paged decode attention, batch %d, ctx %d, 16 q / 8 kv "
                         "heads, head_dim 128, block_size 16, FP16 KV for `value`" % (B, CTX),
             "partition_size": f16["partition_size"], "partitions": f16["partitions"],
             "waves_per_workgroup": lib.pa_get_decode_waves(),
+            "kv_dtype": "f16 (fp8-e4m3 reported beside it under `fp8`)", "q_dtype": "f16", "accumulate": "f32",
         },
         "pct_hbm_peak": round(100.0 * f16["gbps"] / HBM_PEAK_GBPS, 2),
         "us_per_step": round(f16["us_per_step"], 2),
