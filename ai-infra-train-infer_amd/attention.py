@@ -6,6 +6,7 @@ runner that binds caches by isinstance() and sets the global context can use the
 unchanged.  Everything computes on the GPU through libpaged_attn.so; a CPU tensor or a
 missing library raises RuntimeError (there is no fallback path).
 """
+import functools
 from typing import Optional
 
 import torch
@@ -372,36 +373,80 @@ def _workspace(device, nbytes):
     return ws
 
 
-# Workgroups the decode launch should reach before it stops splitting the context: one
-# 4-wave workgroup per CU (256 CUs) already keeps 8 KiB per wave in flight on every SIMD, and a
-# launch of that size runs as a single round with no merge pass (measured: splitting the
-# batch-64 / ctx-4096 launch further only adds the merge and the partial traffic).
-_TARGET_WORKGROUPS = 256
-_MIN_AUTO_PARTITION = 256
+# ---- how a decode launch is shaped ------------------------------------------------------------
+# Two rates bound a launch: what HBM delivers to the whole GPU, and what one CU can pull however
+# many workgroups it hosts (about 1.3 x its 1/256 share).  Workgroups are dealt to CUs in rounds,
+# so the launch lasts as long as its busiest CU needs: 288 equal workgroups on 256 CUs make two
+# rounds, not 1.125.  The context is split where the larger of the two bounds, plus about 2 us per
+# round of workgroups and 5 us + 0.25 us per partition for the merge pass, is smallest.  The rates
+# are measurements on an MI355X (batch 4..128, contexts 2k..32k, fp16 and fp8 caches).
+_MIN_AUTO_PARTITION = 256          # tokens
+_MAX_AUTO_PARTITIONS = 128
+_HBM_BYTES_PER_NS = 6050.0
+_CU_BYTES_PER_NS = {2: 31.0, 1: 22.0}      # by cache element size: fp8 rows cost more arithmetic per byte
+_ROUND_NS = 2000.0
+_MERGE_NS = (5000.0, 250.0)        # fixed, per partition (the pass itself and the partials it re-reads)
+_DEFAULT_COMPUTE_UNITS = 256
+_CU_COUNT = {}
 
 
-def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2):
-    """Partition size for a decode launch that has no caller-given one.
+def _compute_units(device):
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    n = _CU_COUNT.get(idx)
+    if n is None:
+        n = torch.cuda.get_device_properties(idx).multi_processor_count or _DEFAULT_COMPUTE_UNITS
+        _CU_COUNT[idx] = n
+    return n
 
-    One workgroup serves the query heads of one KV head (two heads of a GQA group at a time),
-    or of two adjacent KV heads when a head's row is 128 bytes or less.  If batch x those head
-    groups already give _TARGET_WORKGROUPS workgroups the launch is a single pass; otherwise the
-    context is split into power-of-two partitions of at least 256 tokens until about that many
-    exist.  Returns (partition_size, max_partitions); (0, 1) means a single pass.
-    """
+
+def pairs_kv_heads(workgroups, narrow_rows, can_pair, compute_units=_DEFAULT_COMPUTE_UNITS):
+    """The launch's own rule (pa_decode) for serving two adjacent KV heads from one workgroup:
+    always for rows of 128 bytes or less, otherwise when halving the `workgroups` of the unpaired
+    launch does not add a round (fewer, longer-lived workgroups stream better)."""
+    if not can_pair:
+        return False
+    if narrow_rows or workgroups >= 8 * compute_units:
+        return True
+    rounds = -(-workgroups // compute_units)
+    paired_rounds = -(-workgroups // (2 * compute_units))
+    return 2 * paired_rounds <= rounds
+
+
+@functools.lru_cache(maxsize=4096)
+def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2,
+                     compute_units=_DEFAULT_COMPUTE_UNITS):
+    """Partition size for a decode launch that has no caller-given one: the split of
+    `max_context` (a multiple of 16 tokens, at least 256) with the smallest modelled time.
+    Returns (partition_size, max_partitions); (0, 1) means a single pass."""
     g = num_q_heads // num_kv_heads
     gc = 2 if g % 2 == 0 else 1
-    hpw = 2 if (head_dim * kv_elem_bytes <= 128 and g == gc and num_kv_heads % 2 == 0) else 1
-    units = batch * (num_q_heads // (gc * hpw))
-    if units >= _TARGET_WORKGROUPS or max_context <= _MIN_AUTO_PARTITION:
-        return 0, 1
-    p = _MIN_AUTO_PARTITION
-    while p * 2 < max_context and units * ((max_context + 2 * p - 1) // (2 * p)) >= _TARGET_WORKGROUPS:
-        p *= 2
-    parts = (max_context + p - 1) // p
-    if parts <= 1:
-        return 0, 1
-    return p, parts
+    can_pair = g == gc and num_kv_heads % 2 == 0
+    narrow = head_dim * kv_elem_bytes <= 128
+    units = batch * (num_q_heads // gc)                  # workgroups of one partition, unpaired
+    token_bytes = 2.0 * head_dim * kv_elem_bytes         # K and V of one head
+    cu_rate = _CU_BYTES_PER_NS.get(kv_elem_bytes, 31.0)
+    hbm_ns = batch * num_kv_heads * max_context * token_bytes / _HBM_BYTES_PER_NS
+    best = None
+    max_parts = max(1, min(_MAX_AUTO_PARTITIONS, max_context // _MIN_AUTO_PARTITION))
+    seen = set()
+    for want in range(1, max_parts + 1):
+        psize = -(-max_context // want)
+        psize = -(-psize // 16) * 16
+        parts = -(-max_context // psize)
+        if parts in seen:
+            continue
+        seen.add(parts)
+        wgs = units * parts
+        heads = 2 if pairs_kv_heads(wgs, narrow, can_pair, compute_units) else 1
+        rounds = -(-(wgs // heads) // compute_units)
+        busiest_ns = rounds * min(psize, max_context) * heads * token_bytes / cu_rate
+        cost = max(hbm_ns, busiest_ns) + rounds * _ROUND_NS
+        if parts > 1:
+            cost += _MERGE_NS[0] + _MERGE_NS[1] * parts
+        if best is None or cost < best[0] * 0.99:        # ties go to the coarser split
+            best = (cost, psize, parts)
+    _, psize, parts = best
+    return (0, 1) if parts <= 1 else (psize, parts)
 
 
 def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale=None,
@@ -440,7 +485,7 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale
     max_context = tables.shape[1] * block_size
     if partition_size is None:
         psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim,
-                                        k_cache.element_size())
+                                        k_cache.element_size(), _compute_units(q.device))
     else:
         psize = int(partition_size)
         parts = max(1, (max_context + psize - 1) // psize)
@@ -626,7 +671,7 @@ class PartitionedPagedAttention(PagedAttention):
         if self.adaptive:
             max_context = ctx.block_tables.shape[1] * self.k_cache.shape[1]
             auto, _ = choose_partition(q.shape[0], self.num_heads, self.num_kv_heads, max_context,
-                                       self.head_dim, self.k_cache.element_size())
+                                       self.head_dim, self.k_cache.element_size(), _compute_units(q.device))
             if auto == 0 or auto >= psize:
                 psize = None          # the launch's own choice: single pass or coarser partitions
         return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,

@@ -47,16 +47,23 @@ def test_cpu_tensors_are_refused_not_emulated(pa):
 
 
 def test_choose_partition_policy(pa):
-    # headline shape: 64 x 8 head groups = 512 workgroups fill the GPU on their own -> single pass
+    # headline shape: 64 x 4 pairs of KV heads = one workgroup per CU -> single pass
     assert pa.choose_partition(64, 16, 8, 4096) == (0, 1)
-    # a quarter of that batch is split four ways
+    # a quarter of that batch: split so that a workgroup exists for every CU
     p, n = pa.choose_partition(16, 16, 8, 4096)
-    assert p % 16 == 0 and n == (4096 + p - 1) // p and 16 * 8 * n >= 256
-    # long context, tiny batch: many partitions, each at least 256 tokens
+    assert p % 16 == 0 and n == (4096 + p - 1) // p and n > 1 and 16 * 8 * n >= 256
+    # long context, tiny batch: partitions of at least 256 tokens, close to one workgroup per CU
     p, n = pa.choose_partition(4, 16, 8, 32768)
-    assert p >= 256 and n * p >= 32768
+    assert p >= 256 and p % 16 == 0 and n * p >= 32768 and 192 <= 4 * 8 * n <= 512
+    # 36 sequences x 8 heads = 288 workgroups would take two rounds in a single pass: split instead
+    p, n = pa.choose_partition(36, 16, 8, 8192)
+    assert n > 1
     # short context never splits
     assert pa.choose_partition(1, 16, 8, 256) == (0, 1)
+    # the pairing rule the launch applies: narrow rows always, wide rows when it adds no round
+    f = pa.attention.pairs_kv_heads
+    assert f(512, False, True) and not f(256, False, True) and f(288, False, True) and not f(600, False, True)
+    assert f(100, True, True) and not f(512, False, False) and f(4096, False, True)
 
 
 def test_block_pool_layout(pa):
