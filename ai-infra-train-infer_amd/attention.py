@@ -418,6 +418,8 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
     """Partition size for a decode launch that has no caller-given one: the split of
     `max_context` (a multiple of 16 tokens, at least 256) with the smallest modelled time.
     Returns (partition_size, max_partitions); (0, 1) means a single pass."""
+    if max_context <= _MIN_AUTO_PARTITION or batch <= 0:
+        return 0, 1
     g = num_q_heads // num_kv_heads
     gc = 2 if g % 2 == 0 else 1
     can_pair = g == gc and num_kv_heads % 2 == 0
