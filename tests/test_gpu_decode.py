@@ -243,3 +243,24 @@ def test_partitioned_module_adaptive_and_exact_splits_agree(pa, gpu, adaptive):
         got = attn._decode_attention(d["q"], pa.get_context()).cpu()
         pa.reset_context()
         check(got, oracle_decode(c), "fp16")
+
+
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+@pytest.mark.parametrize("pair_mode", [0, 1, 2])
+@pytest.mark.parametrize("lens", [[2999, 301, 1777], [4100] * 5, [257, 5003], [1200] * 12, [33, 2000, 640, 3100, 90, 1500, 2111]])
+def test_launch_policy_splits_and_head_pairing_keep_the_result(pa, lib, gpu, cache, pair_mode, lens):
+    """The launch's own choices - partition sizes that are multiples of 16 rather than powers of
+    two, one or two KV heads per wave - never show in the output."""
+    c = cases.make_case(sum(lens) % 97, lens, sum((n + 15) // 16 for n in lens) + 7, cache=cache)
+    want = oracle_decode(c)
+    psize, parts = pa.choose_partition(len(lens), 16, 8, c["block_tables"].shape[1] * 16, 128, 1 if cache == "fp8" else 2)
+    assert psize % 16 == 0 and (parts == 1 or parts * psize >= max(lens))
+    assert lib.pa_set_decode_pair_heads(pair_mode) == 0
+    try:
+        got = gpu_decode(pa, c, gpu)
+        odd = gpu_decode(pa, c, gpu, partition_size=16 * 23)       # 368 tokens: neither a power of two nor a block multiple of 8 tiles
+    finally:
+        lib.pa_set_decode_pair_heads(1)
+    check(got, want, cache)
+    check(odd, want, cache)
+    assert lib.pa_set_decode_pair_heads(3) != 0 and lib.pa_set_decode_pair_heads(-1) != 0
