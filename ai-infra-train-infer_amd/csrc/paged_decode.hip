@@ -128,7 +128,9 @@ struct Tile {
 // HPW = KV heads per wavefront.  With HPW == 2 the 8-lane row groups alternate between two
 // adjacent KV heads, so 16 consecutive lanes read 2 x (head_dim * element size) contiguous
 // bytes: rows of 128 bytes or less (fp8 at head_dim 128, anything at head_dim 64) are then
-// fetched as 256-byte pieces, which HBM serves about 10% faster than lone 128-byte lines.
+// fetched as 256-byte pieces, which HBM serves about 10% faster than lone 128-byte lines; wider
+// rows gain from it when it lets the launch run as fewer, longer-lived workgroups (the launch
+// code decides).
 template <int KV, int D, int GC, int W, int HPW>
 __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams p) {
   using G = Geo<KV, D, HPW>;
