@@ -28,13 +28,13 @@ from .attention import (
     HAS_FLASH_ATTN,
     HAS_TRITON,
 )
-from .model_runner import ModelRunner, ModelRunnerConfig
+from .model_runner import ModelRunner, ModelRunnerConfig, DecodeState
 from .qwen3_paged import Qwen3PagedConfig, Qwen3PagedModel
 from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "slot_mapping", "add_rms_norm", "silu_mul", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "DecodeState", "slot_mapping", "add_rms_norm", "silu_mul", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",

@@ -44,6 +44,44 @@ __global__ __launch_bounds__(256) void slot_mapping_kernel(const int64_t* __rest
   slots[t] = slot;
 }
 
+// One decode step of a batch whose metadata lives on the device: every active row (context
+// length > 0) gets one token longer, a row whose new token opens a block receives that block's id
+// from new_blocks, and position and slot of the new token follow from the row's own table.  One
+// thread per row; rows do not interact.
+__global__ __launch_bounds__(256) void decode_advance_kernel(int32_t* __restrict__ block_tables, int64_t bt_stride,
+                                                             int32_t* __restrict__ context_lens,
+                                                             int64_t* __restrict__ positions,
+                                                             int32_t* __restrict__ slots,
+                                                             const int32_t* __restrict__ new_blocks,
+                                                             int64_t* __restrict__ input_ids,
+                                                             const int64_t* __restrict__ next_tokens,
+                                                             int32_t* __restrict__ fresh, int batch,
+                                                             int table_width, int block_size, int num_blocks) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= batch) return;
+  const int len = context_lens[r];
+  if (len <= 0) {            // inactive row: writes nothing, reads nothing
+    slots[r] = -1;
+    positions[r] = 0;
+    return;
+  }
+  // the token to feed: what the last step produced for this row, unless the row has just been
+  // admitted and still holds the token its prefill produced
+  if (fresh && fresh[r]) fresh[r] = 0;
+  else if (next_tokens && input_ids) input_ids[r] = next_tokens[r];
+  const int pos = len;       // index of the token being written; the context then counts it
+  const int col = pos / block_size;
+  int32_t block = -1;
+  if (col < table_width) {
+    int32_t* entry = block_tables + (int64_t)r * bt_stride + col;
+    if (new_blocks && new_blocks[r] >= 0) *entry = new_blocks[r];
+    block = *entry;
+  }
+  context_lens[r] = len + 1;
+  positions[r] = pos;
+  slots[r] = (block >= 0 && block < num_blocks) ? block * block_size + pos % block_size : -1;
+}
+
 }  // namespace pa
 
 using namespace pa;
@@ -67,4 +105,23 @@ extern "C" int pa_slot_mapping(const int64_t* positions, const int32_t* cu_seqle
                      cu_seqlens_q, block_tables, bt_stride, slots, num_tokens, (int)num_rows, (int)table_width,
                      (int)block_size, (int)num_blocks);
   return check_launch("pa_slot_mapping");
+}
+
+extern "C" int pa_decode_advance(int32_t* block_tables, int64_t bt_stride, int32_t* context_lens, int64_t* positions,
+                                 int32_t* slots, const int32_t* new_blocks, int64_t* input_ids,
+                                 const int64_t* next_tokens, int32_t* fresh, int64_t batch, int64_t table_width,
+                                 int64_t block_size, int64_t num_blocks, void* stream) {
+  if (batch < 0 || table_width < 0 || block_size <= 0 || num_blocks <= 0)
+    return fail(PA_ERR_BAD_ARG, "pa_decode_advance: negative or zero size");
+  if (batch == 0) return PA_OK;
+  if (!block_tables || !context_lens || !positions || !slots)
+    return fail(PA_ERR_BAD_ARG, "pa_decode_advance: null pointer");
+  if (next_tokens && !input_ids) return fail(PA_ERR_BAD_ARG, "pa_decode_advance: next_tokens without input_ids");
+  if (bt_stride < table_width) return fail(PA_ERR_BAD_ARG, "pa_decode_advance: table stride smaller than its width");
+  if (batch > INT32_MAX || table_width > INT32_MAX || num_blocks * block_size > INT32_MAX)
+    return fail(PA_ERR_UNSUPPORTED, "pa_decode_advance: slots must fit int32");
+  hipLaunchKernelGGL(decode_advance_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     block_tables, bt_stride, context_lens, positions, slots, new_blocks, input_ids, next_tokens,
+                     fresh, (int)batch, (int)table_width, (int)block_size, (int)num_blocks);
+  return check_launch("pa_decode_advance");
 }

@@ -15,7 +15,11 @@ same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_t
   * graph replay copies into static device buffers and pads with slot -1 / context 0, exactly as
     the reference does, but capture needs no host synchronisation inside the model;
   * `run_batch_decode` gets its slot mapping from a kernel instead of two `.item()` reads per
-    sequence, so a decode step driven by device-resident tables never waits for the GPU.
+    sequence, so a decode step driven by device-resident tables never waits for the GPU;
+  * `DecodeState` keeps block tables, context lengths, positions, slots and input ids of the
+    running batch on the GPU between steps: a step uploads at most one block id per sequence
+    (the block its new token opens) and advances everything else with one small kernel, and the
+    graphs recorded over it (`capture_decode_state_graphs`) replay without a single input copy.
 
 HF-model KV gathering and mock logits are outside this path and are not rebuilt.
 """
@@ -52,6 +56,147 @@ def slots_for_range(block_table, start, end, block_size):
     return (bt[pos // block_size] * block_size + pos % block_size).astype(np.int32)
 
 
+class DecodeState:
+    """Decode metadata of up to `max_batch` sequences, resident on the GPU between steps.
+
+    What prepare_decode rebuilds and uploads every step (src/inference/model_runner.py:542-588,
+    814-828) lives here in fixed tensors: `block_tables` [max_batch, max_blocks] int32 (-1 =
+    unused), `context_lens` [max_batch] int32 (0 = free row), `positions` int64, `slot_mapping`
+    int32, `input_ids` int64.  A sequence occupies one row from `admit` (after its prefill) to
+    `retire`; `step` makes every active row one token longer.  Free rows are inert in the
+    kernels (slot -1, context 0), so any prefix [0, n) with n >= `rows_in_use` is a valid batch,
+    which is what graph replay needs.  The host keeps only counters (lengths, tables) to know
+    when a sequence needs its next block; it never reads the device tensors back.
+    """
+
+    def __init__(self, max_batch: int, max_blocks_per_seq: int, block_size: int, num_blocks: int,
+                 device: str = "cuda"):
+        dev = torch.device(device)
+        self.max_batch, self.max_blocks = int(max_batch), int(max_blocks_per_seq)
+        self.block_size, self.num_blocks = int(block_size), int(num_blocks)
+        self.block_tables = torch.full((max_batch, max_blocks_per_seq), -1, dtype=torch.int32, device=dev)
+        self.context_lens = torch.zeros(max_batch, dtype=torch.int32, device=dev)
+        self.positions = torch.zeros(max_batch, dtype=torch.long, device=dev)
+        self.slot_mapping = torch.full((max_batch,), -1, dtype=torch.int32, device=dev)
+        self.input_ids = torch.zeros(max_batch, dtype=torch.long, device=dev)
+        self._new_blocks = torch.full((max_batch,), -1, dtype=torch.int32, device=dev)
+        self._fresh = torch.zeros(max_batch, dtype=torch.int32, device=dev)   # 1: admitted since the last step
+        # two pinned staging buffers used in turn; an event marks when the copy out of one is done
+        self._stage = [[torch.full((max_batch,), -1, dtype=torch.int32).pin_memory(), None] for _ in range(2)]
+        self._turn = 0
+        self._fresh_rows = set()                        # host copy of the same
+        self._lens = [0] * max_batch                    # tokens in the cache, per row (0 = free)
+        self._tables = [[] for _ in range(max_batch)]   # block ids, per row
+
+    @property
+    def rows_in_use(self) -> int:
+        """One past the highest active row."""
+        for r in range(self.max_batch - 1, -1, -1):
+            if self._lens[r] > 0:
+                return r + 1
+        return 0
+
+    def active_rows(self) -> List[int]:
+        return [r for r in range(self.max_batch) if self._lens[r] > 0]
+
+    def num_tokens(self, row: int) -> int:
+        return self._lens[row]
+
+    def admit(self, block_table: List[int], num_cached_tokens: int, next_token: int) -> int:
+        """Give a prefilled sequence (its `num_cached_tokens` tokens are in the cache, `next_token`
+        is the one sampled from the prefill) the lowest free row; returns the row."""
+        if num_cached_tokens <= 0:
+            raise RuntimeError("DecodeState.admit: a sequence enters decode with at least one cached token")
+        if len(block_table) > self.max_blocks or len(block_table) * self.block_size < num_cached_tokens:
+            raise RuntimeError("DecodeState.admit: block table does not fit the state or the tokens")
+        try:
+            row = self._lens.index(0)
+        except ValueError:
+            raise RuntimeError("DecodeState.admit: all %d rows are in use" % self.max_batch) from None
+        host_row = torch.full((self.max_blocks,), -1, dtype=torch.int32)
+        host_row[:len(block_table)] = torch.tensor(block_table, dtype=torch.int32)
+        self.block_tables[row].copy_(host_row.pin_memory(), non_blocking=True)
+        self.context_lens[row].fill_(int(num_cached_tokens))
+        self.input_ids[row].fill_(int(next_token))
+        self._fresh[row].fill_(1)
+        self._fresh_rows.add(row)
+        self._lens[row] = int(num_cached_tokens)
+        self._tables[row] = list(block_table)
+        return row
+
+    def retire(self, row: int) -> List[int]:
+        """Free a row; returns the block ids the sequence held."""
+        self.context_lens[row].fill_(0)
+        self._fresh_rows.discard(row)
+        blocks, self._tables[row], self._lens[row] = self._tables[row], [], 0
+        return blocks
+
+    def rows_needing_block(self) -> List[int]:
+        """Active rows whose next token opens a block they do not have yet."""
+        bs = self.block_size
+        return [r for r in range(self.max_batch)
+                if self._lens[r] > 0 and self._lens[r] % bs == 0 and self._lens[r] // bs >= len(self._tables[r])]
+
+    def step(self, new_blocks: Optional[Dict[int, int]] = None, next_tokens: Optional[torch.Tensor] = None):
+        """Advance every active row by one token.  new_blocks: {row: block id} for the rows of
+        rows_needing_block(); next_tokens: device int64 [>= rows_in_use], row r's entry being the
+        token the previous step produced for row r (the sampler's output as it is); rows admitted
+        since that step keep the token they were admitted with."""
+        from . import _native
+        lib = _native.load()
+        n = self.rows_in_use
+        if next_tokens is not None:
+            next_tokens = next_tokens.reshape(-1)
+            if not next_tokens.is_cuda or next_tokens.dtype != torch.long or not next_tokens.is_contiguous():
+                raise RuntimeError("DecodeState.step: next_tokens must be a contiguous int64 GPU tensor")
+            fed = [r for r in range(n) if self._lens[r] > 0 and r not in self._fresh_rows]
+            if fed and fed[-1] >= next_tokens.numel():
+                raise RuntimeError("DecodeState.step: next_tokens has no entry for row %d" % fed[-1])
+            if next_tokens.numel() < self.max_batch:      # the kernel indexes it by row
+                padded = torch.zeros(self.max_batch, dtype=torch.long, device=next_tokens.device)
+                padded[:next_tokens.numel()] = next_tokens
+                next_tokens = padded
+        missing = [r for r in self.rows_needing_block() if not new_blocks or r not in new_blocks]
+        if missing:
+            raise RuntimeError("DecodeState.step: rows %s need a new block" % missing)
+        new_ptr = None
+        if new_blocks:
+            host, event = self._stage[self._turn]
+            if event is not None:
+                event.synchronize()                       # the copy that last read this buffer
+            host.fill_(-1)
+            for row, block in new_blocks.items():
+                if self._lens[row] <= 0 or len(self._tables[row]) >= self.max_blocks:
+                    raise RuntimeError("DecodeState.step: row %d cannot take a block" % row)
+                host[row] = int(block)
+                self._tables[row].append(int(block))
+            self._new_blocks.copy_(host, non_blocking=True)
+            done = torch.cuda.Event()
+            done.record()
+            self._stage[self._turn][1] = done
+            self._turn ^= 1
+            new_ptr = self._new_blocks.data_ptr()
+        stream = torch.cuda.current_stream(self.block_tables.device).cuda_stream
+        rc = lib.pa_decode_advance(self.block_tables.data_ptr(), self.block_tables.stride(0),
+                                   self.context_lens.data_ptr(), self.positions.data_ptr(),
+                                   self.slot_mapping.data_ptr(), new_ptr, self.input_ids.data_ptr(),
+                                   next_tokens.data_ptr() if next_tokens is not None else None,
+                                   self._fresh.data_ptr(), self.max_batch, self.max_blocks,
+                                   self.block_size, self.num_blocks, stream)
+        _native.check(rc, "pa_decode_advance")
+        for r in range(self.max_batch):
+            if self._lens[r] > 0:
+                self._lens[r] += 1
+        self._fresh_rows.clear()
+
+    def set_context(self, batch: Optional[int] = None):
+        """Point the attention layers at the first `batch` rows (default: the rows in use)."""
+        n = self.rows_in_use if batch is None else batch
+        set_context(False, slot_mapping=self.slot_mapping[:n], context_lens=self.context_lens[:n],
+                    block_tables=self.block_tables[:n])
+        return n
+
+
 class ModelRunner:
     """prepare_prefill / prepare_decode -> run -> logits, around a model that owns
     PagedAttention layers."""
@@ -68,6 +213,7 @@ class ModelRunner:
         self._graph_pool = None
         self._graph_vars: Optional[Dict[str, torch.Tensor]] = None
         self._graph_batch_sizes: List[int] = []
+        self._state_graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
 
     # ---------------------------------------------------------------- cache binding
 
@@ -275,8 +421,50 @@ class ModelRunner:
         self._graphs[graph_bs].replay()
         return self._graph_outputs[graph_bs][:bs]
 
+    # ---------------------------------------------------------------- decode over a DecodeState
+
+    @torch.inference_mode()
+    def capture_decode_state_graphs(self, state: DecodeState, batch_sizes: Optional[List[int]] = None):
+        """Record the decode forward over the first n rows of `state` for each n: the graph's
+        inputs are the state's own tensors, so a replay needs no copies at all."""
+        if not torch.cuda.is_available() or self.model is None:
+            return
+        if batch_sizes is None:
+            batch_sizes = sorted({b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < state.max_batch}
+                                 | {state.max_batch})
+        for bs in sorted(batch_sizes, reverse=True):
+            state.set_context(bs)
+            self.model(state.input_ids[:bs], positions=state.positions[:bs])     # sizes workspaces
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                out = self.model(state.input_ids[:bs], positions=state.positions[:bs])
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            self._state_graphs[(id(state), bs)] = (graph, out)
+            torch.cuda.synchronize()
+            reset_context()
+
+    @torch.inference_mode()
+    def run_decode_state(self, state: DecodeState) -> torch.Tensor:
+        """Logits [rows_in_use, vocab] of the step `state.step()` has just prepared."""
+        if self.model is None:
+            raise RuntimeError("ModelRunner.run_decode_state: no model bound")
+        n = state.rows_in_use
+        if self.config.enable_cuda_graph:
+            sizes = sorted(bs for (sid, bs) in self._state_graphs if sid == id(state) and bs >= n)
+            if sizes:
+                graph, out = self._state_graphs[(id(state), sizes[0])]
+                graph.replay()
+                return out[:n]
+        state.set_context(n)
+        logits = self.model(state.input_ids[:n], positions=state.positions[:n])
+        reset_context()
+        return logits
+
     def invalidate_cuda_graphs(self):
         """Drop every recorded graph (after a weight update)."""
+        self._state_graphs.clear()
         self._graphs.clear()
         self._graph_outputs.clear()
         self._graph_pool = None

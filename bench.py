@@ -292,7 +292,8 @@ def sampler_times(pa, torch, dev, steps, warmup):
 def model_step_cfg5b(pa, torch, dev, steps, warmup):
     """Fifth benchmark configuration, second half: one decode step of a Qwen3-0.6B-shaped model
     (28 layers, hidden 1024, 16q/8kv x 128, random weights) at batch 64, context 2048, FP16 KV:
-    metadata preparation + forward, eagerly and as a replayed HIP graph."""
+    metadata preparation + forward, eagerly and as a replayed HIP graph; then the whole step
+    (advance, forward, greedy sampling) with the metadata kept on the GPU."""
     cfg = pa.Qwen3PagedConfig()
     B, CTX, BS = 64, 2048, 16
     torch.manual_seed(11)
@@ -320,6 +321,46 @@ def model_step_cfg5b(pa, torch, dev, steps, warmup):
         ms, _ = time_steps(torch, step, steps, warmup)
         out[name + "_ms"] = round(ms, 3)
         runner.invalidate_cuda_graphs()
+    # The same step with the metadata resident on the GPU (DecodeState): advance kernel + a graph
+    # over the state's own tensors + greedy sampling on the device, the sampled tokens feeding
+    # the next step without leaving the GPU.  The sequences enter 15 tokens short of a block
+    # boundary so that the timed steps need no new block.
+    runner = pa.ModelRunner(model, pa.ModelRunnerConfig(
+        num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
+        head_dim=cfg.head_dim, hidden_size=cfg.hidden_size, block_size=BS, max_num_blocks=CTX // BS,
+        device="cuda:0", enable_cuda_graph=True, max_cuda_graph_batch_size=B))
+    runner.bind_kv_cache(pool.kv_cache_tensor)
+    state = pa.DecodeState(B, CTX // BS, BS, nb, device=dev)
+    for b in range(B):
+        state.admit(seqs[b]["block_table"], CTX - 15, 1)
+    runner.capture_decode_state_graphs(state, [B])
+    nxt = [None]
+
+    def state_step():
+        state.step(None, nxt[0])
+        nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
+
+    import time as _time
+    n_steps = 12
+    state_step()
+    state_step()
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    host = 0.0
+    for _ in range(n_steps):
+        h0 = _time.perf_counter()
+        state.step(None, nxt[0])
+        host += _time.perf_counter() - h0
+        nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
+    torch.cuda.synchronize()
+    out["device_state_step_ms"] = round((_time.perf_counter() - t0) * 1e3 / n_steps, 3)
+    out["device_state_host_us_per_step"] = round(host * 1e6 / n_steps, 1)
+    t0 = _time.perf_counter()
+    for _ in range(20):
+        runner.prepare_decode(seqs)
+    out["prepare_decode_host_us_per_step"] = round((_time.perf_counter() - t0) * 1e6 / 20, 1)
+    torch.cuda.synchronize()
+    runner.invalidate_cuda_graphs()
     kv_bytes = cfg.num_layers * B * CTX * cfg.num_kv_heads * cfg.head_dim * 2 * 2
     out["kv_bytes_per_step"] = kv_bytes
     out["kv_gbps_in_graph_step"] = round(kv_bytes / out["hip_graph_ms"] / 1e6, 1)

@@ -244,6 +244,26 @@ int pa_sample(const void* logits, int dtype, int64_t row_stride, int64_t batch, 
               float temperature, float top_p, const float* uniforms, int64_t* out, void* stream);
 
 /*
+ * One decode step of a batch whose metadata stays on the device.  For every row r with
+ * context_lens[r] > 0: if new_blocks (optional, int32 [batch], -1 = none) holds a block id for the
+ * row it is stored at block_tables[r][context_lens[r] / block_size] (the block the new token
+ * opens); then positions[r] = context_lens[r] (int64, the new token's index), slots[r] = its
+ * cache slot from the row's table (-1 when outside the table or the pool), and context_lens[r]
+ * grows by one, so that it counts the token being written as the attention kernels expect.
+ * With next_tokens (optional, int64 [batch], e.g. the sampler's output of the step before) the
+ * row's input_ids[r] becomes next_tokens[r] - unless fresh[r] (optional, int32 [batch]) is set:
+ * a row admitted since the last step keeps the token its prefill produced, and the flag is cleared.
+ * Rows with context_lens[r] <= 0 are inactive: slots[r] = -1, positions[r] = 0, nothing else changes.
+ * Replaces: the per-step host loops and uploads of ModelRunner.prepare_decode and
+ * _prepare_block_tables (src/inference/model_runner.py:542-588, 814-828: one Python assignment
+ * per table entry and five fresh device tensors per step).
+ */
+int pa_decode_advance(int32_t* block_tables, int64_t bt_stride, int32_t* context_lens, int64_t* positions,
+                      int32_t* slots, const int32_t* new_blocks, int64_t* input_ids, const int64_t* next_tokens,
+                      int32_t* fresh, int64_t batch, int64_t table_width, int64_t block_size,
+                      int64_t num_blocks, void* stream);
+
+/*
  * One decoder block's residual add fused with the RMSNorm that follows it, one row per token:
  *     s = x + delta            rounded to `dtype` (skipped when delta == NULL: s = x)
  *     normed = weight * (s * rsqrt(mean(s^2) + eps))      fp32, rounded once to `dtype`
