@@ -139,7 +139,8 @@ class DecodeState:
 
     def step(self, new_blocks: Optional[Dict[int, int]] = None, next_tokens: Optional[torch.Tensor] = None):
         """Advance every active row by one token.  new_blocks: {row: block id} for the rows of
-        rows_needing_block(); next_tokens: device int64 [>= rows_in_use], row r's entry being the
+        rows_needing_block(), and for rows whose last block has just been replaced by a private
+        copy (copy-on-write): the id lands in the table column the new token falls into; next_tokens: device int64 [>= rows_in_use], row r's entry being the
         token the previous step produced for row r (the sampler's output as it is); rows admitted
         since that step keep the token they were admitted with."""
         from . import _native
@@ -166,10 +167,14 @@ class DecodeState:
                 event.synchronize()                       # the copy that last read this buffer
             host.fill_(-1)
             for row, block in new_blocks.items():
-                if self._lens[row] <= 0 or len(self._tables[row]) >= self.max_blocks:
+                if self._lens[row] <= 0 or self._lens[row] // self.block_size >= self.max_blocks:
                     raise RuntimeError("DecodeState.step: row %d cannot take a block" % row)
                 host[row] = int(block)
-                self._tables[row].append(int(block))
+                col = self._lens[row] // self.block_size          # the block the new token falls into
+                if col < len(self._tables[row]):
+                    self._tables[row][col] = int(block)          # copy-on-write: a private copy replaces it
+                else:
+                    self._tables[row].append(int(block))
             self._new_blocks.copy_(host, non_blocking=True)
             done = torch.cuda.Event()
             done.record()
