@@ -399,13 +399,14 @@ def _compute_units(device):
     return n
 
 
-def pairs_kv_heads(workgroups, narrow_rows, can_pair, compute_units=_DEFAULT_COMPUTE_UNITS):
+def pairs_kv_heads(workgroups, can_pair, compute_units=_DEFAULT_COMPUTE_UNITS):
     """The launch's own rule (pa_decode) for serving two adjacent KV heads from one workgroup:
-    always for rows of 128 bytes or less, otherwise when halving the `workgroups` of the unpaired
-    launch does not add a round (fewer, longer-lived workgroups stream better)."""
+    when halving the `workgroups` of the unpaired launch does not add a round of them over the
+    CUs (fewer, longer-lived workgroups stream better; with one workgroup or less per CU pairing
+    would only idle CUs)."""
     if not can_pair:
         return False
-    if narrow_rows or workgroups >= 8 * compute_units:
+    if workgroups >= 8 * compute_units:
         return True
     rounds = -(-workgroups // compute_units)
     paired_rounds = -(-workgroups // (2 * compute_units))
@@ -439,10 +440,12 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
             continue
         seen.add(parts)
         wgs = units * parts
-        heads = 2 if pairs_kv_heads(wgs, narrow, can_pair, compute_units) else 1
+        heads = 2 if pairs_kv_heads(wgs, can_pair, compute_units) else 1
+        # lone rows of 128 bytes or less stream about 10% below the rest
+        hbm = hbm_ns * (1.12 if narrow and heads == 1 else 1.0)
         rounds = -(-(wgs // heads) // compute_units)
         busiest_ns = rounds * min(psize, max_context) * heads * token_bytes / cu_rate
-        cost = max(hbm_ns, busiest_ns) + rounds * _ROUND_NS
+        cost = max(hbm, busiest_ns) + rounds * _ROUND_NS
         if parts > 1:
             cost += _MERGE_NS[0] + _MERGE_NS[1] * parts
         if best is None or cost < best[0] * 0.99:        # ties go to the coarser split

@@ -626,20 +626,18 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
 
   hipStream_t st = (hipStream_t)stream;
   // Two adjacent KV heads per wave (each KV head's query group must be handled whole, so that
-  // adjacent workgroup heads are adjacent KV heads): always when one head's row is 128 bytes or
-  // less, where a lone row is too short a read.  For wider rows when halving the workgroups does
-  // not add a round of them over the CUs: a CU streams at a fixed rate however many workgroups
-  // it hosts, the launch takes as long as its busiest CU, and fewer, longer-lived workgroups
-  // stream better (185 -> 178 us at batch 64 / ctx 4096, fp16).
-  const int es = kv == KV_FP8 ? 1 : 2;
+  // adjacent workgroup heads are adjacent KV heads) when halving the workgroups does not add a
+  // round of them over the CUs: a CU streams at a fixed rate however many workgroups it hosts,
+  // the launch takes as long as its busiest CU, and fewer, longer-lived workgroups stream better
+  // (185 -> 178 us at batch 64 / ctx 4096, fp16; rows of 128 bytes or less gain another 10% from
+  // being read as 256-byte pieces).  With a workgroup or less per CU pairing would only idle CUs.
   const bool can_pair = g == gc && num_kv_heads % 2 == 0;
-  const bool narrow = head_dim * es <= 128;
   bool pair = false;
   if (can_pair && g_decode_pair_heads != 0) {
     const int64_t cus = compute_units();
     const int64_t wgs = (num_q_heads / gc) * max_partitions * batch;      // unpaired
     const int64_t rounds = (wgs + cus - 1) / cus, paired_rounds = (wgs + 2 * cus - 1) / (2 * cus);
-    pair = g_decode_pair_heads == 2 || narrow || wgs >= 8 * cus || 2 * paired_rounds <= rounds;
+    pair = g_decode_pair_heads == 2 || wgs >= 8 * cus || 2 * paired_rounds <= rounds;
   }
   const int hpw = pair ? 2 : 1;
   dim3 grid((unsigned)(num_q_heads / (gc * hpw)), (unsigned)max_partitions, (unsigned)batch);

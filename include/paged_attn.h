@@ -320,11 +320,9 @@ int pa_copy_blocks(void* pool, int64_t num_planes, int64_t plane_stride_bytes, i
 /* Tunables of the decode launch (waves per workgroup: 1, 2, 4 or 8). Returns PA_OK or BAD_ARG. */
 int pa_set_decode_waves(int waves_per_workgroup);
 int pa_get_decode_waves(void);
-/* Tunable: one wavefront serves two adjacent KV heads.  0 never; 1 (default) when a head's row
- * is <= 128 bytes (fp8 at head_dim 128, any dtype at head_dim 64), and for wider rows when
- * halving the workgroups does not add a round of them over the CUs; 2 whenever the head layout
- * allows it (whole query groups per workgroup, an even number of KV heads).
- * Returns PA_OK or BAD_ARG. */
+/* Tunable: one wavefront serves two adjacent KV heads.  0 never; 1 (default) when halving the
+ * workgroups does not add a round of them over the CUs; 2 whenever the head layout allows it
+ * (whole query groups per workgroup, an even number of KV heads).  Returns PA_OK or BAD_ARG. */
 int pa_set_decode_pair_heads(int mode);
 /* Tunable of the prefill launch: waves per workgroup, 4 (64 query tokens x 2 heads per K/V tile)
  * or 8 (128 x 2), or 0 = chosen per launch from the grid size (default). Returns PA_OK or BAD_ARG. */

@@ -60,10 +60,10 @@ def test_choose_partition_policy(pa):
     assert n > 1
     # short context never splits
     assert pa.choose_partition(1, 16, 8, 256) == (0, 1)
-    # the pairing rule the launch applies: narrow rows always, wide rows when it adds no round
+    # the pairing rule the launch applies: whenever it adds no round
     f = pa.attention.pairs_kv_heads
-    assert f(512, False, True) and not f(256, False, True) and f(288, False, True) and not f(600, False, True)
-    assert f(100, True, True) and not f(512, False, False) and f(4096, False, True)
+    assert f(512, True) and not f(256, True) and f(288, True) and not f(600, True)
+    assert not f(100, True) and not f(512, False) and f(4096, True)
 
 
 def test_block_pool_layout(pa):
