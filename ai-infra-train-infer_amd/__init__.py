@@ -20,6 +20,7 @@ from .attention import (
     qk_norm_rope_store,
     sample_tokens,
     slot_mapping,
+    gather_kv_cache,
     add_rms_norm,
     silu_mul,
     paged_decode,
@@ -34,7 +35,7 @@ from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "DecodeState", "slot_mapping", "add_rms_norm", "silu_mul", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "DecodeState", "slot_mapping", "gather_kv_cache", "add_rms_norm", "silu_mul", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_prefill", "choose_partition",
     "HAS_FLASH_ATTN", "HAS_TRITON",

@@ -52,6 +52,7 @@ SIGNATURES = {
     "pa_copy_blocks": (_int, [_ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "pa_add_rms_norm": (_int, [_ptr, _i64, _ptr, _i64, _ptr, _int, _f32, _ptr, _i64, _ptr, _i64, _int, _i64, _i64, _ptr]),
     "pa_silu_mul": (_int, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _i64, _i64, _ptr]),
+    "pa_gather_kv": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_decode_advance": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_set_decode_waves": (_int, [_int]),

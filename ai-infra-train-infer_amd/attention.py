@@ -258,6 +258,32 @@ def sample_tokens(logits, temperature=0.7, top_p=0.9, uniforms=None, generator=N
     return out
 
 
+def gather_kv_cache(k_cache, v_cache, block_tables, context_lens, out_len, len_offset=1):
+    """Dense, head-major copies of the paged K and V of a batch:
+    (k, v) each [batch, kv_heads, out_len, head_dim] in the cache's own dtype, rows at or past
+    context_lens - len_offset zero.  One layer of ModelRunner._load_kv_from_paged_cache
+    (src/inference/model_runner.py:340-420) without its host loops."""
+    _require_gpu(k_cache, "gather_kv_cache")
+    _check_cache(k_cache, v_cache, "gather_kv_cache")
+    lib = _native.load()
+    num_blocks, block_size, num_kv_heads, head_dim = k_cache.shape
+    if block_tables.dim() != 2 or context_lens.numel() != block_tables.shape[0]:
+        raise RuntimeError("gather_kv_cache: block_tables [batch, max_blocks] and context_lens [batch] expected")
+    tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+    if tables.stride(1) != 1:
+        tables = tables.contiguous()
+    lens = _int32(context_lens, "gather_kv_cache")
+    batch = tables.shape[0]
+    k_out = torch.empty((batch, num_kv_heads, int(out_len), head_dim), dtype=k_cache.dtype, device=k_cache.device)
+    v_out = torch.empty_like(k_out)
+    rc = lib.pa_gather_kv(k_cache.data_ptr(), v_cache.data_ptr(), tables.data_ptr(), tables.stride(0), tables.shape[1],
+                          lens.data_ptr(), int(len_offset), k_out.data_ptr(), v_out.data_ptr(), batch, num_kv_heads,
+                          head_dim, k_cache.element_size(), block_size, num_blocks, int(out_len),
+                          _stream_ptr(k_cache.device))
+    _native.check(rc, "pa_gather_kv")
+    return k_out, v_out
+
+
 def _rows2d(t, what):
     """[rows, width] view whose rows are 16-byte aligned and unit-stride inside; (tensor, row stride)."""
     if t.dim() != 2:

@@ -21,7 +21,10 @@ same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_t
     (the block its new token opens) and advances everything else with one small kernel, and the
     graphs recorded over it (`capture_decode_state_graphs`) replay without a single input copy.
 
-HF-model KV gathering and mock logits are outside this path and are not rebuilt.
+The reference's shipped mode around a HuggingFace model (`bind_hf_model`, `_hf_prefill_forward`,
+`_hf_decode_forward`, `_store_hf_*`, `_load_kv_from_paged_cache`, :118-462) is here too, with its
+per-entry slot loops and index gathers replaced by one gather kernel per layer.  Mock logits (a
+runner without a model) are not rebuilt.
 """
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
@@ -219,6 +222,7 @@ class ModelRunner:
         self._graph_vars: Optional[Dict[str, torch.Tensor]] = None
         self._graph_batch_sizes: List[int] = []
         self._state_graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._hf_model: Optional[torch.nn.Module] = None
 
     # ---------------------------------------------------------------- cache binding
 
@@ -331,6 +335,8 @@ class ModelRunner:
 
     @torch.inference_mode()
     def run(self, input_ids, positions, is_prefill=True):
+        if self._hf_model is not None:
+            return self._run_hf_model(input_ids, positions, is_prefill)
         if self.model is None:
             raise RuntimeError("ModelRunner.run: no model bound")
         use_graph = (not is_prefill and self.config.enable_cuda_graph and self._graph_vars is not None
@@ -357,6 +363,117 @@ class ModelRunner:
         slots = slot_mapping(positions, block_tables, self.block_size, num_blocks)
         set_context(is_prefill=False, slot_mapping=slots, context_lens=context_lens, block_tables=block_tables)
         return self.run(input_ids, positions, is_prefill=False)
+
+    # ---------------------------------------------------------------- HuggingFace-style models
+    # The reference's shipped kv_cache mode (src/inference/model_runner.py:118-462): the model is
+    # a HuggingFace causal LM that knows nothing of paging; its K/V are written into the paged pool
+    # after the forward and rebuilt from the pool as past_key_values before every decode step.
+    # Same methods and call order; the pool traffic goes through pa_kv_store and pa_gather_kv.
+
+    def bind_hf_model(self, model: torch.nn.Module):
+        self._hf_model = model
+
+    def _run_hf_model(self, input_ids, positions, is_prefill):
+        ctx = get_context()
+        if is_prefill:
+            logits = self._hf_prefill_forward(input_ids, positions, ctx)
+        else:
+            logits = self._hf_decode_forward(input_ids, positions, ctx)
+        reset_context()
+        return logits
+
+    def _hf_prefill_forward(self, input_ids, positions, ctx):
+        """One sequence [num_tokens]: full forward, K/V of every layer into the pool, logits
+        [num_tokens, vocab] (model_runner.py:192-230)."""
+        ids2 = input_ids.unsqueeze(0) if input_ids.dim() == 1 else input_ids
+        pos2 = positions.unsqueeze(0) if positions.dim() == 1 else positions
+        mask = torch.ones(1, ids2.shape[1], dtype=torch.long, device=input_ids.device)
+        outputs = self._hf_model(input_ids=ids2, position_ids=pos2, attention_mask=mask, use_cache=True)
+        if ctx.slot_mapping is not None and self._kv_cache is not None:
+            self._store_hf_kv_to_paged_cache(outputs.past_key_values, ctx.slot_mapping)
+        return outputs.logits.squeeze(0)
+
+    def _hf_decode_forward(self, input_ids, positions, ctx):
+        """One token per sequence: past_key_values gathered from the pool, single-token forward,
+        the new token's K/V into the pool, logits [batch, vocab] (model_runner.py:232-285)."""
+        ids2 = input_ids.unsqueeze(1) if input_ids.dim() == 1 else input_ids
+        pos2 = positions.unsqueeze(1) if positions.dim() == 1 else positions
+        past, mask = None, None
+        if ctx.context_lens is not None:
+            max_past_len = int(ctx.context_lens.max().item()) - 1       # the reference's one host read
+            past = self._load_kv_from_paged_cache(ctx.block_tables, ctx.context_lens, max_past_len)
+            mask = torch.ones(ids2.shape[0], max_past_len + 1, dtype=torch.long, device=input_ids.device)
+        outputs = self._hf_model(input_ids=ids2, position_ids=pos2, attention_mask=mask,
+                                 past_key_values=past, use_cache=True)
+        if ctx.slot_mapping is not None and self._kv_cache is not None:
+            self._store_hf_decode_kv_to_cache(outputs.past_key_values, ctx)
+        return outputs.logits.squeeze(1)
+
+    def _pool_layer(self, layer_idx):
+        if self._k_scale is not None or self._kv_cache.element_size() == 1:
+            raise RuntimeError("the HuggingFace path stores K/V unscaled: bind an fp16 or bf16 pool")
+        return self._kv_cache[0, layer_idx], self._kv_cache[1, layer_idx]
+
+    def _store_hf_kv_to_paged_cache(self, past_key_values, slot_mapping):
+        """Prefill: [1, kv_heads, seq, dim] per layer -> the slots of the sequence
+        (model_runner.py:287-312)."""
+        from .attention import store_kv_cache
+        for layer_idx in range(self.config.num_layers):
+            k, v = self._extract_layer_kv(past_key_values, layer_idx)
+            k_cache, v_cache = self._pool_layer(layer_idx)
+            k = k.squeeze(0).transpose(0, 1).contiguous().to(k_cache.dtype)
+            v = v.squeeze(0).transpose(0, 1).contiguous().to(v_cache.dtype)
+            store_kv_cache(k, v, k_cache, v_cache, slot_mapping)
+
+    def _store_hf_decode_kv_to_cache(self, past_key_values, ctx):
+        """Decode: the last position of [batch, kv_heads, past + 1, dim] per layer -> each
+        sequence's new slot (model_runner.py:314-338)."""
+        from .attention import store_kv_cache
+        for layer_idx in range(self.config.num_layers):
+            k, v = self._extract_layer_kv(past_key_values, layer_idx)
+            k_cache, v_cache = self._pool_layer(layer_idx)
+            k_new = k[:, :, -1, :].contiguous().to(k_cache.dtype)        # [batch, kv_heads, dim]
+            v_new = v[:, :, -1, :].contiguous().to(v_cache.dtype)
+            store_kv_cache(k_new, v_new, k_cache, v_cache, ctx.slot_mapping)
+
+    def _load_kv_from_paged_cache(self, block_tables, context_lens, max_past_len: Optional[int] = None):
+        """past_key_values for a decode step: per layer K, V [batch, kv_heads, max_past_len, dim]
+        with each sequence's first context_len - 1 positions from the pool and zeros after
+        (model_runner.py:340-420).  None when there is no cache or nothing cached yet.  Returned
+        as a transformers DynamicCache when that class is importable, else as a tuple of (K, V)."""
+        from .attention import gather_kv_cache
+        if self._kv_cache is None or block_tables is None or context_lens is None:
+            return None
+        if max_past_len is None:
+            max_past_len = int(context_lens.max().item()) - 1
+        if max_past_len <= 0:
+            return None
+        layers = []
+        for layer_idx in range(self.config.num_layers):
+            k_cache, v_cache = self._pool_layer(layer_idx)
+            layers.append(gather_kv_cache(k_cache, v_cache, block_tables, context_lens, max_past_len, len_offset=1))
+        try:
+            from transformers import DynamicCache
+            cache = DynamicCache()
+            for layer_idx, (k, v) in enumerate(layers):
+                cache.update(k, v, layer_idx)
+            return cache
+        except ImportError:
+            return tuple(layers)
+
+    @staticmethod
+    def _extract_layer_kv(past_key_values, layer_idx: int):
+        """(K, V) of one layer, each [batch, kv_heads, seq, dim], from the cache classes of
+        transformers 5.x (.layers) and 4.x (.key_cache) or a legacy tuple (model_runner.py:435-462)."""
+        if hasattr(past_key_values, "layers"):
+            layer = past_key_values.layers[layer_idx]
+            return layer.keys, layer.values
+        if hasattr(past_key_values, "key_cache"):
+            return past_key_values.key_cache[layer_idx], past_key_values.value_cache[layer_idx]
+        layer_kv = past_key_values[layer_idx]
+        if isinstance(layer_kv, (tuple, list)):
+            return layer_kv[0], layer_kv[1]
+        raise ValueError("Unsupported past_key_values format: %s" % type(past_key_values))
 
     # ---------------------------------------------------------------- sampling
 

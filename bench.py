@@ -183,6 +183,23 @@ def kv_store_times(pa, torch, dev, steps, warmup):
     return out
 
 
+def kv_gather_times(pa, torch, dev, steps, warmup):
+    """Paged cache -> dense head-major past_key_values of one layer (what the reference's
+    HuggingFace mode rebuilds every decode step): batch 64, context 2048, 8 KV heads x 128, fp16.
+    Microseconds, and the achieved bandwidth over the bytes read plus the bytes written."""
+    B, CTX, HKV, D, BS = 64, 2048, 8, 128, 16
+    g = torch.Generator(device=dev).manual_seed(13)
+    nb = B * (CTX // BS) + 8
+    kc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+    vc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
+    tables = torch.randperm(nb, generator=g, device=dev)[:B * (CTX // BS)].view(B, -1).to(torch.int32).contiguous()
+    lens = torch.full((B,), CTX, dtype=torch.int32, device=dev)
+    ms, _ = time_steps(torch, lambda: pa.gather_kv_cache(kc, vc, tables, lens, CTX - 1), steps, warmup)
+    moved = 2 * 2 * B * (CTX - 1) * HKV * D * 2            # K and V, read and written
+    return {"workload": "64 x 2047 past tokens, 8 kv heads x 128, fp16, one layer", "us": round(ms * 1e3, 1),
+            "bytes_read_plus_written": moved, "gbps": round(moved / ms / 1e6, 1)}
+
+
 def fused_qk_times(pa, torch, dev, steps, warmup):
     """Per-head q/k RMSNorm + rotary embedding + paged cache write of one layer: the fused kernel
     beside the same steps as separate torch ops followed by store_kv_cache, for one decode step
@@ -513,6 +530,7 @@ def main():
     line["prefill_mfma"] = prefill
     if not args.no_extras:
         line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
+        line["kv_gather"] = kv_gather_times(pa, torch, dev, args.steps, args.warmup)
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
         line["block_elementwise"] = block_elementwise_times(pa, torch, dev, args.steps, args.warmup)
         line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)

@@ -244,6 +244,22 @@ int pa_sample(const void* logits, int dtype, int64_t row_stride, int64_t batch, 
               float temperature, float top_p, const float* uniforms, int64_t* out, void* stream);
 
 /*
+ * Gather the paged K and V of a batch into dense head-major tensors
+ *     k_out, v_out  [batch, num_kv_heads, out_len, head_dim]   (same element type as the cache)
+ * out[b, h, pos] = cache[slot(b, pos), h] for pos < context_lens[b] - len_offset, zeros after
+ * that (and for positions whose table entry lies outside the table or the pool); slot(b, pos) =
+ * block_tables[b][pos / block_size] * block_size + pos % block_size.  Bytes are moved as they are
+ * (elem_bytes 1, 2 or 4; head_dim * elem_bytes a multiple of 16; 16-byte aligned bases).
+ * Replaces: ModelRunner._load_kv_from_paged_cache (src/inference/model_runner.py:340-420), one
+ * layer of it: the per-entry Python slot loop, the index gather, the zeroing of the padding and
+ * the transposing copy.  len_offset = 1 there (the token being decoded is not part of the past).
+ */
+int pa_gather_kv(const void* k_cache, const void* v_cache, const int32_t* block_tables, int64_t bt_stride,
+                 int64_t table_width, const int32_t* context_lens, int64_t len_offset, void* k_out, void* v_out,
+                 int64_t batch, int64_t num_kv_heads, int64_t head_dim, int64_t elem_bytes, int64_t block_size,
+                 int64_t num_blocks, int64_t out_len, void* stream);
+
+/*
  * One decode step of a batch whose metadata stays on the device.  For every row r with
  * context_lens[r] > 0: if new_blocks (optional, int32 [batch], -1 = none) holds a block id for the
  * row it is stored at block_tables[r][context_lens[r] / block_size] (the block the new token

@@ -5,6 +5,7 @@ metadata (TEST INFRASTRUCTURE ONLY; plain Python loops, lists out):
   decode_metadata    src/inference/model_runner.py:542-588
   block_tables       src/inference/model_runner.py:814-828
   batch_decode_slots src/inference/model_runner.py:670-682
+  load_kv_from_paged_cache  src/inference/model_runner.py:340-420 (one layer, tensors in / out)
 
 Pinned by the closed form "slot of position p = block_table[p // BS] * BS + p % BS" in
 tests/test_model_runner_host.py.
@@ -86,3 +87,30 @@ def batch_decode_slots(positions, block_tables, block_size):
             continue
         slots.append(block_tables[i][block_idx] * block_size + offset)
     return slots
+
+
+def load_kv_from_paged_cache(k_cache, v_cache, block_tables, context_lens):
+    """src/inference/model_runner.py:361-420 for one layer: slot of every (sequence, past
+    position) by the double loop, gather, zero the rows past each sequence's past length,
+    [batch, len, heads, dim] -> [batch, heads, len, dim].  Returns None when nothing is cached,
+    as the reference does."""
+    import torch
+    num_blocks, block_size, num_kv_heads, head_dim = k_cache.shape
+    batch = len(block_tables)
+    past_lens = [int(n) - 1 for n in context_lens]
+    max_past_len = max(past_lens) if past_lens else 0
+    if max_past_len <= 0:
+        return None
+    k_flat = k_cache.reshape(num_blocks * block_size, num_kv_heads, head_dim)
+    v_flat = v_cache.reshape(num_blocks * block_size, num_kv_heads, head_dim)
+    slot_indices = torch.zeros(batch, max_past_len, dtype=torch.long)
+    for b in range(batch):
+        for pos in range(max(past_lens[b], 0)):
+            slot_indices[b, pos] = int(block_tables[b][pos // block_size]) * block_size + pos % block_size
+    k_gathered = k_flat[slot_indices.view(-1)].view(batch, max_past_len, num_kv_heads, head_dim).clone()
+    v_gathered = v_flat[slot_indices.view(-1)].view(batch, max_past_len, num_kv_heads, head_dim).clone()
+    for b in range(batch):
+        if past_lens[b] < max_past_len:
+            k_gathered[b, max(past_lens[b], 0):] = 0
+            v_gathered[b, max(past_lens[b], 0):] = 0
+    return k_gathered.transpose(1, 2).contiguous(), v_gathered.transpose(1, 2).contiguous()
