@@ -23,8 +23,8 @@ same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_t
 
 The reference's shipped mode around a HuggingFace model (`bind_hf_model`, `_hf_prefill_forward`,
 `_hf_decode_forward`, `_store_hf_*`, `_load_kv_from_paged_cache`, :118-462) is here too, with its
-per-entry slot loops and index gathers replaced by one gather kernel per layer.  Mock logits (a
-runner without a model) are not rebuilt.
+per-entry slot loops and index gathers replaced by one gather kernel per layer, and so is its mock
+mode (a runner without a model returns random logits).
 """
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
@@ -338,7 +338,12 @@ class ModelRunner:
         if self._hf_model is not None:
             return self._run_hf_model(input_ids, positions, is_prefill)
         if self.model is None:
-            raise RuntimeError("ModelRunner.run: no model bound")
+            # the reference's mock mode (src/inference/model_runner.py:152-158): a runner without a
+            # model answers with random logits, so that a scheduler can be exercised on its own
+            logits = torch.randn(input_ids.shape[0], self.config.vocab_size, device=input_ids.device,
+                                 dtype=torch.float32)
+            reset_context()
+            return logits
         use_graph = (not is_prefill and self.config.enable_cuda_graph and self._graph_vars is not None
                      and any(b >= input_ids.size(0) for b in self._graph_batch_sizes))
         if use_graph:
@@ -354,8 +359,6 @@ class ModelRunner:
         [batch, 1], positions [batch] (of the token being written), block_tables [batch, max_blocks]
         int32, context_lens [batch] int32 (counting that token) -> logits [batch, vocab]
         (src/inference/model_runner.py:639-708)."""
-        if self.model is None:
-            raise RuntimeError("ModelRunner.run_batch_decode: no model bound")
         from .attention import slot_mapping
         if input_ids.dim() == 2:
             input_ids = input_ids.squeeze(1)

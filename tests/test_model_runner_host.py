@@ -90,3 +90,14 @@ def test_no_tables_means_none(pa):
     ctx = pa.get_context()
     assert ctx.slot_mapping is None and ctx.block_tables is None
     pa.reset_context()
+
+
+def test_mock_mode_returns_random_logits_and_resets_the_context(pa):
+    """src/inference/model_runner.py:152-158: no model bound -> random fp32 logits."""
+    import torch
+    r = pa.ModelRunner(None, pa.ModelRunnerConfig(vocab_size=97, device="cpu"))
+    ids, pos = r.prepare_decode([{"token_ids": [1, 2, 3], "block_table": [0]}, {"token_ids": [4], "block_table": [1]}])
+    assert pa.get_context().context_lens is not None
+    logits = r.run(ids, pos, is_prefill=False)
+    assert logits.shape == (2, 97) and logits.dtype == torch.float32
+    assert pa.get_context().context_lens is None
