@@ -199,7 +199,10 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
   // blockIdx.x (fastest, dealt round-robin to the 8 XCDs) is the head group: all query tiles of
   // one KV head then run on the same XCD and share its L2, so a K/V tile is fetched from HBM
   // once instead of once per query tile.
-  const int tok0 = blockIdx.y * BM;
+  // Query tiles are handed out last first: under the causal mask the last tile of a sequence has
+  // the most keys, and when a launch has more workgroups than the GPU holds at once the long ones
+  // should start first and the short ones fill the end.
+  const int tok0 = (int)(gridDim.y - 1 - blockIdx.y) * BM;
   if (tok0 >= lq) return;
   const int shift = lk - lq;  // row i sees keys <= i + shift
 
