@@ -35,6 +35,7 @@
 #include <math.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <type_traits>
 #include <utility>
 
@@ -69,6 +70,7 @@ struct PrefillParams {
 enum : int { SRC_F16 = 0, SRC_BF16 = 1, SRC_FP8 = 2, SRC_F32 = 3 };
 
 constexpr int kBN = 64;  // keys per tile
+constexpr int kMaxDevices = 64;
 
 // LDS reads of the tile loop, issued as opaque asm.  ds_read_b64_tr_b16 is the LDS transpose load
 // of gfx950: within each block of 16 lanes, lane i receives element (i % 4) of the 8 bytes
@@ -553,11 +555,15 @@ template <int D, int HPWG, int SRC, int W>
 static int launch_prefill(const PrefillParams& p, dim3 grid, hipStream_t st) {
   auto kern = paged_prefill_kernel<D, HPWG, SRC, W>;
   const size_t smem = sizeof(PrefillLds<D>);
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
+  // the attribute belongs to the kernel on one device: once per instantiation and device
+  static std::atomic<bool> attr_set[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(PA_ERR_LAUNCH, "pa_prefill: cannot tell the current device");
+  if (!attr_set[dev].load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return fail(PA_ERR_LAUNCH, "pa_prefill: cannot raise the dynamic LDS limit");
-    attr_set = true;
+    attr_set[dev].store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, grid, dim3(64 * W), smem, st, p);
   return PA_OK;
