@@ -34,15 +34,15 @@ SIGNATURES = {
     "pa_kv_store_fp8": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                _i64, _i64, _ptr]),
     "pa_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
-    "pa_decode": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr,
+    "pa_decode": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr, _ptr,
                          _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
-                         _ptr]),
-    "pa_decode_partials": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _ptr,
+                         _int, _int, _int, _ptr]),
+    "pa_decode_partials": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
-                                  _ptr]),
+                                  _int, _int, _int, _ptr]),
     "pa_merge": (_int, [_ptr, _i64, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_prefill": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr,
-                          _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _ptr]),
+                          _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]),
     "pa_fp8_e4m3_to_f32": (_int, [_ptr, _ptr, _i64, _ptr]),
     "pa_f32_to_fp8_e4m3": (_int, [_ptr, _ptr, _i64, _ptr]),
     "pa_qk_norm_rope_store": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _int, _f32, _ptr,
@@ -55,10 +55,7 @@ SIGNATURES = {
     "pa_gather_kv": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_decode_advance": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
-    "pa_set_decode_waves": (_int, [_int]),
-    "pa_get_decode_waves": (_int, []),
-    "pa_set_decode_pair_heads": (_int, [_int]),
-    "pa_set_prefill_waves": (_int, [_int]),
+    "pa_check_tables": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
 }
 
 _lock = threading.Lock()

@@ -7,6 +7,7 @@ unchanged.  Everything computes on the GPU through libpaged_attn.so; a CPU tenso
 missing library raises RuntimeError (there is no fallback path).
 """
 import functools
+import os
 from typing import Optional
 
 import torch
@@ -389,14 +390,70 @@ def slot_mapping(positions, block_tables, block_size, num_blocks, cu_seqlens_q=N
     return out
 
 
-def _workspace(device, nbytes):
-    """Per (device, stream) scratch for the partition partials; grows, never shrinks."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _WORKSPACES[key] = ws
+def _device_index(device):
+    return device.index if device.index is not None else torch.cuda.current_device()
+
+
+def reserve_decode_workspace(device, nbytes):
+    """Make the device's partition workspace at least `nbytes` large and return it.
+
+    One workspace per device serves every partitioned decode launch on it.  It only grows, and
+    a tensor it has outgrown is kept alive, never handed back to the allocator: a HIP graph
+    recorded earlier still holds that tensor's address.  Growing allocates, so it must happen
+    outside a graph capture - whoever captures decode graphs reserves the largest size first
+    (ModelRunner does, from its largest batch and the launch policy's partition limit); inside a
+    capture a workspace that is too small raises instead of allocating from the graph's pool.
+    Launches that run at the same time on different streams of one device must not share it: give
+    those their own tensor through paged_decode(workspace=...)."""
+    idx = _device_index(device)
+    held = _WORKSPACES.setdefault(idx, [])
+    if held and held[-1].numel() >= nbytes:
+        return held[-1]
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            "paged_decode: the partition workspace of cuda:%d holds %d bytes and this launch needs %d; "
+            "it cannot grow during a graph capture - call reserve_decode_workspace() before capturing"
+            % (idx, held[-1].numel() if held else 0, nbytes))
+    ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=torch.device("cuda", idx))
+    held.append(ws)
     return ws
+
+
+def decode_workspace_bytes(batch, num_q_heads, head_dim, max_partitions=None):
+    """Bytes of partition workspace that cover any launch of up to `batch` rows: by default for the
+    finest split the launch policy ever chooses."""
+    parts = _MAX_AUTO_PARTITIONS if max_partitions is None else int(max_partitions)
+    return _native.load().pa_workspace_bytes(int(batch), int(num_q_heads), int(head_dim), parts)
+
+
+def release_decode_workspaces():
+    """Drop every partition workspace.  Only safe once no recorded graph that used one will be
+    replayed again."""
+    _WORKSPACES.clear()
+
+
+def check_block_tables(block_tables, context_lens, block_size, num_blocks):
+    """(entries outside the pool, rows whose context outruns the table), counted on the GPU over the
+    part of each row that a decode launch would read.  The attention kernels clamp both instead of
+    faulting, so a corrupt table shows up as wrong numbers; this is the check that names it.
+    Synchronises with the host: a debugging aid (PA_DEBUG_TABLES=1 runs it before every decode)."""
+    _require_gpu(block_tables, "check_block_tables")
+    lib = _native.load()
+    tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+    if tables.stride(1) != 1:
+        tables = tables.contiguous()
+    lens = _int32(context_lens, "check_block_tables")
+    counts = torch.zeros(2, dtype=torch.int32, device=tables.device)
+    rc = lib.pa_check_tables(tables.data_ptr(), tables.stride(0), tables.shape[1], lens.data_ptr(),
+                             tables.shape[0], int(block_size), int(num_blocks), counts.data_ptr(),
+                             _stream_ptr(tables.device))
+    _native.check(rc, "pa_check_tables")
+    bad, short = counts.tolist()
+    return bad, short
+
+
+def _debug_tables():
+    return os.environ.get("PA_DEBUG_TABLES", "0") not in ("", "0")
 
 
 # ---- how a decode launch is shaped ------------------------------------------------------------
@@ -480,13 +537,27 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
     return (0, 1) if parts <= 1 else (psize, parts)
 
 
+def choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2,
+                  compute_units=_DEFAULT_COMPUTE_UNITS):
+    """(partition_size, max_partitions, kv_heads_per_wave) of a decode launch that has no
+    caller-given shape; kv_heads_per_wave 0 leaves the choice between one and two KV heads per
+    wave to the launch itself (the rule of pairs_kv_heads)."""
+    psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, kv_elem_bytes,
+                                    compute_units)
+    return psize, parts, 0
+
+
 def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale=None,
-                 v_scale=None, partition_size=None, out=None):
+                 v_scale=None, partition_size=None, out=None, waves=0, kv_heads_per_wave=None,
+                 q_heads_per_wave=0, workspace=None):
     """Decode attention of q [batch, heads, head_dim] against the paged cache.
 
     partition_size None: single pass, or an automatic split when the batch alone cannot fill
     the GPU (same result up to fp32 rounding).  partition_size > 0: the partitioned algorithm
     of src/inference/attention.py:434-626 with that size.  Never synchronises with the host.
+    waves / kv_heads_per_wave / q_heads_per_wave shape the launch (0 or None: the launch policy's
+    choice); they never change the result.  workspace: a uint8 tensor for the partition partials
+    instead of the device's shared one.
     """
     _require_gpu(q, "paged_decode")
     _require_gpu(k_cache, "paged_decode")
@@ -513,30 +584,45 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale
     fp8 = kv_code == _native.DTYPE_FP8_E4M3
     if fp8 and (k_scale is None or v_scale is None):
         raise RuntimeError("paged_decode: fp8 cache needs k_scale and v_scale")
+    if _debug_tables():
+        bad, short = check_block_tables(tables, lens, block_size, num_blocks)
+        if bad or short:
+            raise RuntimeError("paged_decode: %d block-table entries outside the pool of %d blocks, %d rows whose "
+                               "context_len needs more than the table's %d columns"
+                               % (bad, num_blocks, short, tables.shape[1]))
     max_context = tables.shape[1] * block_size
+    hpw = kv_heads_per_wave
     if partition_size is None:
-        psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim,
-                                        k_cache.element_size(), _compute_units(q.device))
+        psize, parts, auto_hpw = choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim,
+                                               k_cache.element_size(), _compute_units(q.device))
+        if hpw is None:
+            hpw = auto_hpw
     else:
         psize = int(partition_size)
         parts = max(1, (max_context + psize - 1) // psize)
     ws_ptr, ws_bytes = None, 0
     if parts > 1:
         ws_bytes = lib.pa_workspace_bytes(batch, num_q_heads, head_dim, parts)
-        ws = _workspace(q.device, ws_bytes)
+        if workspace is not None:
+            if workspace.dtype != torch.uint8 or not workspace.is_cuda or workspace.numel() < ws_bytes:
+                raise RuntimeError("paged_decode: workspace must be a uint8 GPU tensor of at least %d bytes" % ws_bytes)
+            ws = workspace
+        else:
+            ws = reserve_decode_workspace(q.device, ws_bytes)
         ws_ptr = ws.data_ptr()
     rc = lib.pa_decode(q.data_ptr(), _code(q.dtype, "paged_decode"), qs, k_cache.data_ptr(),
                        v_cache.data_ptr(), k_scale.data_ptr() if fp8 else None,
                        v_scale.data_ptr() if fp8 else None, kv_code, tables.data_ptr(),
-                       tables.stride(0), lens.data_ptr(), out.data_ptr(), out.stride(0), batch,
-                       num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, float(scale),
-                       psize, parts, ws_ptr, ws_bytes, _stream_ptr(q.device))
+                       tables.stride(0), tables.shape[1], lens.data_ptr(), out.data_ptr(), out.stride(0),
+                       batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, float(scale),
+                       psize, parts, ws_ptr, ws_bytes, int(waves or 0), int(hpw or 0),
+                       int(q_heads_per_wave or 0), _stream_ptr(q.device))
     _native.check(rc, "pa_decode")
     return out
 
 
 def paged_prefill(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, scale,
-                  block_tables=None, k_scale=None, v_scale=None, out=None):
+                  block_tables=None, k_scale=None, v_scale=None, out=None, waves=0):
     """Causal varlen prefill attention on the MFMA kernel.
 
     q [total_new_tokens, heads, head_dim]; cu_seqlens_q / cu_seqlens_k int32 [num_seqs + 1]
@@ -544,6 +630,7 @@ def paged_prefill(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, sca
     the paged caches [num_blocks, block_size, kv_heads, head_dim] and row i of a chunk sees the
     cached prefix plus the chunk up to itself; without, they are the dense new-token tensors
     [total_k_tokens, kv_heads, head_dim] (src/inference/attention.py:243-257).
+    waves: 0 = the launch's own choice of waves per workgroup, or 4 / 8; never changes the result.
     """
     _require_gpu(q, "paged_prefill")
     _require_gpu(k_src, "paged_prefill")
@@ -592,7 +679,7 @@ def paged_prefill(q, k_src, v_src, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, sca
                         v_scale.data_ptr() if fp8 else None, kv_code, bt_ptr, bt_stride,
                         cu_q.data_ptr(), cu_k.data_ptr(), out.data_ptr(), out.stride(0), num_seqs,
                         int(max_seqlen_q), num_q_heads, num_kv_heads, head_dim, block_size,
-                        num_blocks, float(scale), _stream_ptr(q.device))
+                        num_blocks, float(scale), int(waves or 0), _stream_ptr(q.device))
     _native.check(rc, "pa_prefill")
     return out
 

@@ -584,18 +584,9 @@ static int launch_prefill_hpwg(const PrefillParams& p, dim3 grid, int hpwg, int 
   return hpwg == 2 ? launch_prefill_src<D, 2, W>(p, grid, src, st) : launch_prefill_src<D, 1, W>(p, grid, src, st);
 }
 
-static int g_prefill_waves = 0;  // 0 = chosen per launch
-
 }  // namespace pa
 
 using namespace pa;
-
-extern "C" int pa_set_prefill_waves(int waves) {
-  if (waves != 0 && waves != 4 && waves != 8)
-    return fail(PA_ERR_BAD_ARG, "pa_set_prefill_waves: waves per workgroup must be 0 (automatic), 4 or 8");
-  g_prefill_waves = waves;
-  return PA_OK;
-}
 
 extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                           const void* v_cache, const float* k_scale, const float* v_scale,
@@ -603,7 +594,10 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, void* out,
                           int64_t out_token_stride, int64_t num_seqs, int64_t max_seqlen_q,
                           int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
-                          int64_t block_size, int64_t num_blocks, float scale, void* stream) {
+                          int64_t block_size, int64_t num_blocks, float scale,
+                          int waves_per_workgroup, void* stream) {
+  if (waves_per_workgroup != 0 && waves_per_workgroup != 4 && waves_per_workgroup != 8)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill: waves_per_workgroup must be 0 (automatic), 4 or 8");
   if (num_seqs < 0 || max_seqlen_q < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
     return fail(PA_ERR_BAD_ARG, "pa_prefill: negative or zero size");
   if (num_seqs == 0 || max_seqlen_q == 0) return PA_OK;
@@ -655,7 +649,7 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
   const int hpwg = (g % 2 == 0) ? 2 : 1;
   // 8 waves per workgroup share each K/V tile between twice as many query rows, which halves
   // the bytes every CU pulls through its L1; worth it once such workgroups fill most of the chip.
-  int w = g_prefill_waves;
+  int w = waves_per_workgroup;
   if (w == 0) {
     const int64_t bm8 = 256 / hpwg;
     const int64_t wgs8 = (num_q_heads / hpwg) * ((max_seqlen_q + bm8 - 1) / bm8) * num_seqs;

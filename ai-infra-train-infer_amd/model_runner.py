@@ -501,6 +501,7 @@ class ModelRunner:
         self._graph_batch_sizes = sorted(batch_sizes)
         max_bs = max(batch_sizes)
         dev = self.config.device
+        self._reserve_decode_workspace(max_bs)
         gv = {
             "input_ids": torch.zeros(max_bs, dtype=torch.long, device=dev),
             "positions": torch.zeros(max_bs, dtype=torch.long, device=dev),
@@ -512,7 +513,7 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
                         block_tables=gv["block_tables"][:bs])
-            # warm-up outside the capture: allocates the partition workspace and library handles
+            # warm-up outside the capture: library handles, allocator warm-up
             self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
             torch.cuda.synchronize()
             with torch.cuda.graph(graph, pool=self._graph_pool):
@@ -524,6 +525,15 @@ class ModelRunner:
             torch.cuda.synchronize()
             reset_context()
         self._graph_vars = gv
+
+    def _reserve_decode_workspace(self, max_batch):
+        """Size the device's partition workspace for the finest split any decode launch of up to
+        max_batch rows can choose, before anything is recorded: a workspace never grows inside a
+        capture, and one that a graph has recorded is never freed."""
+        from .attention import decode_workspace_bytes, reserve_decode_workspace
+        cfg = self.config
+        reserve_decode_workspace(torch.device(cfg.device),
+                                 decode_workspace_bytes(max_batch, cfg.num_heads, cfg.head_dim))
 
     def _run_with_cuda_graph(self, input_ids, positions):
         bs = input_ids.size(0)
@@ -557,9 +567,10 @@ class ModelRunner:
         if batch_sizes is None:
             batch_sizes = sorted({b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < state.max_batch}
                                  | {state.max_batch})
+        self._reserve_decode_workspace(max(batch_sizes))
         for bs in sorted(batch_sizes, reverse=True):
             state.set_context(bs)
-            self.model(state.input_ids[:bs], positions=state.positions[:bs])     # sizes workspaces
+            self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):

@@ -44,7 +44,7 @@ extern "C" {
 #define PA_DTYPE_F32 2
 #define PA_DTYPE_FP8_E4M3 3 /* OCP e4m3fn, the layout of torch.float8_e4m3fn */
 
-/* Library ABI version (bumped when a signature changes). */
+/* Library ABI version (bumped when a signature changes); 2 = launch shape as per-call arguments. */
 int pa_version(void);
 
 /* Message for the last non-zero return code on this thread ("" if none). */
@@ -116,18 +116,36 @@ int64_t pa_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t head_dim,
  *   q_dtype              PA_DTYPE_F16 / BF16 / F32 (out has the same type)
  *   kv_dtype             PA_DTYPE_F16 / BF16 / FP8_E4M3
  *   k_scale, v_scale     required for fp8, ignored otherwise
+ *   block_tables         rows bt_stride entries apart, table_width (<= bt_stride) of them valid
+ *                        columns: a context that needs more columns than that re-reads the last
+ *                        one instead of running off the row (pa_check_tables counts such rows)
  *   num_blocks           blocks in the pool (block ids are clamped to it)
  *   head_dim             64 or 128;  block_size a power of two >= 8
+ *   num_q_heads          any multiple of num_kv_heads; all query heads of a KV head are served
+ *                        by one workgroup (so its K/V rows leave HBM once) when the ratio is
+ *                        1, 2, 4, 8 or 16, by ratio/4, ratio/2 or ratio workgroups otherwise
  *   partition_size       a multiple of 16 (ignored when max_partitions == 1)
  *   workspace            >= pa_workspace_bytes(...) bytes, 256-byte aligned
+ *   waves_per_workgroup  0 = the launch's own choice, or 1, 2, 4, 8
+ *   kv_heads_per_wave    0 = the launch's own choice (1 or 2), or 1, 2, 4, 8: adjacent KV heads
+ *                        read by one wavefront, i.e. contiguous pieces of that many head rows per
+ *                        token.  More than one needs num_q_heads / num_kv_heads <= 2 and a
+ *                        num_kv_heads it divides; 4 and 8 also need a ratio of 2 and 4 or 8 waves
+ *                        (PA_ERR_UNSUPPORTED otherwise).
+ *   q_heads_per_wave     0 = the launch's own choice, or 1, 2, 4 (a divisor of the GQA ratio):
+ *                        query heads of a KV head held in one wave's registers; the rest of the
+ *                        ratio goes to groups of waves inside the workgroup (factors 2 and 4)
+ *                        and, beyond that, to separate workgroups.
+ *                        The result does not depend on any of the three.
  */
 int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
               const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
-              const int32_t* block_tables, int64_t bt_stride, const int32_t* context_lens,
-              void* out, int64_t out_token_stride, int64_t batch, int64_t num_q_heads,
-              int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
-              float scale, int64_t partition_size, int64_t max_partitions, void* workspace,
-              int64_t workspace_bytes, void* stream);
+              const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
+              const int32_t* context_lens, void* out, int64_t out_token_stride, int64_t batch,
+              int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+              int64_t num_blocks, float scale, int64_t partition_size, int64_t max_partitions,
+              void* workspace, int64_t workspace_bytes, int waves_per_workgroup,
+              int kv_heads_per_wave, int q_heads_per_wave, void* stream);
 
 /*
  * First half of the partitioned decode only: fills `workspace` and does not merge.
@@ -141,10 +159,11 @@ int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, const void* k_
 int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                        const void* v_cache, const float* k_scale, const float* v_scale,
                        int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
-                       const int32_t* context_lens, int64_t batch, int64_t num_q_heads,
-                       int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
-                       int64_t num_blocks, float scale, int64_t partition_size,
+                       int64_t table_width, const int32_t* context_lens, int64_t batch,
+                       int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                       int64_t block_size, int64_t num_blocks, float scale, int64_t partition_size,
                        int64_t max_partitions, void* workspace, int64_t workspace_bytes,
+                       int waves_per_workgroup, int kv_heads_per_wave, int q_heads_per_wave,
                        void* stream);
 
 /*
@@ -179,6 +198,8 @@ int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* cont
  *   head_dim             64 or 128;  block_size a power of two
  *   max_seqlen_q         upper bound of Lq_s (sizes the launch grid)
  *   scale                positive and finite
+ *   waves_per_workgroup  0 = chosen per launch from the grid size, 4 (64 query tokens x 2 heads
+ *                        per K/V tile) or 8 (128 x 2); the result does not depend on it
  */
 int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
@@ -186,7 +207,7 @@ int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, const void* k
                const int32_t* cu_seqlens_k, void* out, int64_t out_token_stride,
                int64_t num_seqs, int64_t max_seqlen_q, int64_t num_q_heads,
                int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
-               float scale, void* stream);
+               float scale, int waves_per_workgroup, void* stream);
 
 /*
  * fp8-e4m3fn -> fp32 conversion of n bytes (the in-register dequant step of the
@@ -333,16 +354,21 @@ int pa_slot_mapping(const int64_t* positions, const int32_t* cu_seqlens_q, const
 int pa_copy_blocks(void* pool, int64_t num_planes, int64_t plane_stride_bytes, int64_t block_bytes,
                    int64_t num_blocks, const int32_t* pairs, int64_t num_pairs, void* stream);
 
-/* Tunables of the decode launch (waves per workgroup: 1, 2, 4 or 8). Returns PA_OK or BAD_ARG. */
-int pa_set_decode_waves(int waves_per_workgroup);
-int pa_get_decode_waves(void);
-/* Tunable: one wavefront serves two adjacent KV heads.  0 never; 1 (default) when halving the
- * workgroups does not add a round of them over the CUs; 2 whenever the head layout allows it
- * (whole query groups per workgroup, an even number of KV heads).  Returns PA_OK or BAD_ARG. */
-int pa_set_decode_pair_heads(int mode);
-/* Tunable of the prefill launch: waves per workgroup, 4 (64 query tokens x 2 heads per K/V tile)
- * or 8 (128 x 2), or 0 = chosen per launch from the grid size (default). Returns PA_OK or BAD_ARG. */
-int pa_set_prefill_waves(int waves_per_workgroup);
+/*
+ * Debug aid for the caller side of the decode path.  The attention kernels never fault on a bad
+ * table: they clamp block ids to the pool and table columns to table_width, which turns a
+ * corrupt table into wrong numbers instead of an error.  This call counts, on the device, what a
+ * decode launch over the same arguments would clamp:
+ *   counts[0] += table entries in the first ceil(context_len / block_size) columns of a row
+ *                that lie outside [0, num_blocks)
+ *   counts[1] += rows whose context needs more than table_width columns
+ * counts is a device int32[2] that the caller clears beforehand and reads afterwards.
+ * No counterpart in the reference, whose host-side indexing raises on such input
+ * (src/inference/attention.py:340-352).
+ */
+int pa_check_tables(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
+                    const int32_t* context_lens, int64_t batch, int64_t block_size,
+                    int64_t num_blocks, int32_t* counts, void* stream);
 
 #ifdef __cplusplus
 }

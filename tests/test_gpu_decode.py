@@ -19,10 +19,10 @@ def oracle_decode(c):
                          c["scale"], c["k_scale"], c["v_scale"], c["cache_dtype"])
 
 
-def gpu_decode(pa, c, gpu, partition_size=None):
+def gpu_decode(pa, c, gpu, partition_size=None, **shape):
     d = cases.to_device(c, gpu)
     out = pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
-                          d["scale"], d["k_scale"], d["v_scale"], partition_size=partition_size)
+                          d["scale"], d["k_scale"], d["v_scale"], partition_size=partition_size, **shape)
     torch.cuda.synchronize()
     return out.cpu()
 
@@ -43,23 +43,40 @@ def test_every_workgroup_width(pa, lib, gpu, waves, cache):
     c = cases.make_case(40 + waves, [1, 15, 16, 17, 100, 333, 512, 47], 128, cache=cache,
                         q_dtype=torch.bfloat16 if cache == "bf16" else torch.float16)
     want = oracle_decode(c)
-    assert lib.pa_set_decode_waves(waves) == 0
-    try:
-        got_single = gpu_decode(pa, c, gpu)
-        got_part = gpu_decode(pa, c, gpu, partition_size=64)
-    finally:
-        lib.pa_set_decode_waves(4)
+    got_single = gpu_decode(pa, c, gpu, waves=waves)
+    got_part = gpu_decode(pa, c, gpu, partition_size=64, waves=waves)
     check(got_single, want, cache)
     check(got_part, want, cache)
 
 
 @pytest.mark.parametrize("hq,hkv,d", [(16, 8, 128), (8, 8, 128), (32, 8, 128), (16, 2, 64),
-                                       (4, 4, 64), (12, 4, 128)])
+                                       (4, 4, 64), (12, 4, 128), (64, 8, 128), (32, 2, 128),
+                                       (24, 4, 128), (40, 8, 64), (48, 4, 64)])
 @pytest.mark.parametrize("cache", ["fp16", "fp8"])
 def test_head_shapes(pa, gpu, hq, hkv, d, cache):
+    """GQA ratios 1, 2, 3, 4, 5, 6, 8, 12 and 16: the map h -> h // G (attention.py:366-370)."""
     c = cases.make_case(hq * 3 + d, [5, 64, 129, 700], 96, num_heads=hq, num_kv_heads=hkv,
                         head_dim=d, cache=cache)
-    check(gpu_decode(pa, c, gpu), oracle_decode(c), cache)
+    want = oracle_decode(c)
+    check(gpu_decode(pa, c, gpu), want, cache)
+    check(gpu_decode(pa, c, gpu, partition_size=128), want, cache)
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (32, 2), (24, 4)])
+@pytest.mark.parametrize("qpw", [1, 2, 4])
+@pytest.mark.parametrize("cache", ["fp16", "fp8", "bf16"])
+def test_query_group_layouts_keep_the_result(pa, gpu, hq, hkv, qpw, cache):
+    """Wide GQA groups: however the query heads of a KV head are spread over a wave's registers,
+    the wave groups of a workgroup and separate workgroups, the output is the same."""
+    if (hq // hkv) % qpw:
+        pytest.skip("q_heads_per_wave must divide the GQA ratio")
+    c = cases.make_case(hq + qpw, [3, 200, 1025, 77], 96, num_heads=hq, num_kv_heads=hkv, cache=cache,
+                        q_dtype=torch.bfloat16 if cache == "bf16" else torch.float16)
+    want = oracle_decode(c)
+    check(gpu_decode(pa, c, gpu, q_heads_per_wave=qpw), want, cache)
+    check(gpu_decode(pa, c, gpu, partition_size=256, q_heads_per_wave=qpw), want, cache)
+    # 4 waves: no split of the query group over wave groups when two heads sit in a wave
+    check(gpu_decode(pa, c, gpu, q_heads_per_wave=qpw, waves=4), want, cache)
 
 
 @pytest.mark.parametrize("bs", [8, 32, 128])
@@ -167,8 +184,9 @@ def test_partials_match_the_reference_partition_outputs(pa, lib, gpu):
     ws = torch.zeros(nbytes, dtype=torch.uint8, device=gpu)
     rc = lib.pa_decode_partials(d["q"].data_ptr(), 2, H * D, d["k_cache"].data_ptr(),
                                 d["v_cache"].data_ptr(), None, None, 0, d["block_tables"].data_ptr(),
-                                d["block_tables"].stride(0), d["context_lens"].data_ptr(), B, H, 8, D,
-                                16, c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, None)
+                                d["block_tables"].stride(0), d["block_tables"].shape[1],
+                                d["context_lens"].data_ptr(), B, H, 8, D,
+                                16, c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, 0, 0, 0, None)
     assert rc == 0, lib.pa_last_error()
     out = torch.empty(B, H, D, dtype=torch.float32, device=gpu)
     rc = lib.pa_merge(ws.data_ptr(), nbytes, d["context_lens"].data_ptr(), out.data_ptr(), 2, H * D,
@@ -202,8 +220,8 @@ def test_more_partitions_than_workspace_rows_still_exact(pa, lib, gpu):
     out = torch.empty(B, H, D, dtype=torch.float16, device=gpu)
     rc = lib.pa_decode(d["q"].data_ptr(), 0, H * D, d["k_cache"].data_ptr(), d["v_cache"].data_ptr(),
                        None, None, 0, d["block_tables"].data_ptr(), d["block_tables"].stride(0),
-                       d["context_lens"].data_ptr(), out.data_ptr(), H * D, B, H, 8, D, 16,
-                       c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, None)
+                       d["block_tables"].shape[1], d["context_lens"].data_ptr(), out.data_ptr(), H * D, B, H, 8, D, 16,
+                       c["num_blocks"], c["scale"], P, parts, ws.data_ptr(), nbytes, 0, 0, 0, None)
     assert rc == 0, lib.pa_last_error()
     torch.cuda.synchronize()
     check(out.cpu(), oracle_decode(c), "fp16")
@@ -214,12 +232,12 @@ def test_c_abi_argument_errors(lib, gpu):
     p = t.data_ptr()
     base = dict(q=p, kc=p, vc=p, bt=p, cl=p, out=p)
     def call(**kw):
-        a = dict(hq=16, hkv=8, d=128, bs=16, psize=0, parts=1, ws=None, wsb=0, kvd=0)
+        a = dict(hq=16, hkv=8, d=128, bs=16, psize=0, parts=1, ws=None, wsb=0, kvd=0, waves=0, hpw=0, qpw=0)
         a.update(kw)
         return lib.pa_decode(base["q"], 0, a["hq"] * a["d"], base["kc"], base["vc"], None, None,
-                             a["kvd"], base["bt"], 1, base["cl"], base["out"], a["hq"] * a["d"], 1,
+                             a["kvd"], base["bt"], 1, 1, base["cl"], base["out"], a["hq"] * a["d"], 1,
                              a["hq"], a["hkv"], a["d"], a["bs"], 4, 1.0, a["psize"], a["parts"],
-                             a["ws"], a["wsb"], None)
+                             a["ws"], a["wsb"], a["waves"], a["hpw"], a["qpw"], None)
     assert call(d=96) == -2 and b"head_dim" in lib.pa_last_error()
     assert call(bs=12) == -2
     assert call(bs=4) == -2
@@ -227,6 +245,10 @@ def test_c_abi_argument_errors(lib, gpu):
     assert call(kvd=3) == -1                      # fp8 without scales
     assert call(parts=4, psize=500, ws=p, wsb=1 << 30) == -2      # not a multiple of 16
     assert call(parts=4, psize=512) == -4         # workspace missing
+    assert call(waves=3) == -1 and call(hpw=3) == -1 and call(qpw=3) == -1
+    assert call(hq=32, hpw=2) == -2               # several KV heads per wave need a GQA ratio <= 2
+    assert call(hq=32, qpw=8) == -1 and call(hq=24, hkv=8, qpw=2) == -2
+    assert call(hpw=4, waves=2) == -2
 
 
 @pytest.mark.parametrize("adaptive", [True, False])
@@ -246,21 +268,92 @@ def test_partitioned_module_adaptive_and_exact_splits_agree(pa, gpu, adaptive):
 
 
 @pytest.mark.parametrize("cache", ["fp16", "fp8"])
-@pytest.mark.parametrize("pair_mode", [0, 1, 2])
+@pytest.mark.parametrize("hpw", [None, 1, 2, 4, 8])
 @pytest.mark.parametrize("lens", [[2999, 301, 1777], [4100] * 5, [257, 5003], [1200] * 12, [33, 2000, 640, 3100, 90, 1500, 2111]])
-def test_launch_policy_splits_and_head_pairing_keep_the_result(pa, lib, gpu, cache, pair_mode, lens):
+def test_launch_policy_splits_and_head_pairing_keep_the_result(pa, lib, gpu, cache, hpw, lens):
     """The launch's own choices - partition sizes that are multiples of 16 rather than powers of
-    two, one or two KV heads per wave - never show in the output."""
+    two, one to eight KV heads per wave - never show in the output."""
     c = cases.make_case(sum(lens) % 97, lens, sum((n + 15) // 16 for n in lens) + 7, cache=cache)
     want = oracle_decode(c)
     psize, parts = pa.choose_partition(len(lens), 16, 8, c["block_tables"].shape[1] * 16, 128, 1 if cache == "fp8" else 2)
     assert psize % 16 == 0 and (parts == 1 or parts * psize >= max(lens))
-    assert lib.pa_set_decode_pair_heads(pair_mode) == 0
-    try:
-        got = gpu_decode(pa, c, gpu)
-        odd = gpu_decode(pa, c, gpu, partition_size=16 * 23)       # 368 tokens: neither a power of two nor a block multiple of 8 tiles
-    finally:
-        lib.pa_set_decode_pair_heads(1)
+    got = gpu_decode(pa, c, gpu, kv_heads_per_wave=hpw)
+    odd = gpu_decode(pa, c, gpu, partition_size=16 * 23, kv_heads_per_wave=hpw)   # 368 tokens: neither a power of two nor a block multiple of 8 tiles
     check(got, want, cache)
     check(odd, want, cache)
-    assert lib.pa_set_decode_pair_heads(3) != 0 and lib.pa_set_decode_pair_heads(-1) != 0
+    if hpw in (4, 8):
+        check(gpu_decode(pa, c, gpu, kv_heads_per_wave=hpw, waves=8), want, cache)
+
+
+def test_table_check_counts_what_the_kernels_would_clamp(pa, gpu, monkeypatch):
+    c = cases.make_case(60, [100, 40, 0, 33], 32)
+    d = cases.to_device(c, gpu)
+    assert pa.check_block_tables(d["block_tables"], d["context_lens"], 16, c["num_blocks"]) == (0, 0)
+    bad = d["block_tables"].clone()
+    bad[0, 2] = c["num_blocks"]          # inside row 0's context (7 blocks): counted
+    bad[1, 1] = -5                        # inside row 1's context (3 blocks): counted
+    bad[1, 5] = -5                        # past row 1's context: never read, not counted
+    bad[2, 0] = 99999                     # padded row: not counted
+    lens = d["context_lens"].clone()
+    lens[3] = 16 * bad.shape[1] + 1       # needs one more column than the table has ...
+    pads = bad.shape[1] - 3               # ... and now covers the -1 padding behind its 3 blocks
+    assert pa.check_block_tables(bad, lens, 16, c["num_blocks"]) == (2 + pads, 1)
+    # the attention launch itself survives such a table (clamped reads) ...
+    out = pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], bad, lens, d["scale"])
+    torch.cuda.synchronize()
+    assert out.shape == d["q"].shape
+    # ... and names it when asked to
+    monkeypatch.setenv("PA_DEBUG_TABLES", "1")
+    with pytest.raises(RuntimeError, match="outside the pool"):
+        pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], bad, lens, d["scale"])
+    got = pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"], d["scale"])
+    check(got.cpu(), oracle_decode(c), "fp16")
+
+
+def test_workspace_is_per_device_grows_outside_captures_and_outlives_graphs(pa, gpu):
+    """A partitioned launch recorded in a graph keeps its workspace address: a later, larger
+    launch grows the workspace without freeing the recorded one, and growth inside a capture is
+    an error instead of an allocation from the graph's pool."""
+    pa.release_decode_workspaces()
+    small = cases.make_case(61, [3000, 2000], 2 * 188 + 8)
+    d = cases.to_device(small, gpu)
+    want = oracle_decode(small)
+    out = torch.empty_like(d["q"])
+
+    def run_small():
+        pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                        d["scale"], partition_size=256, out=out)
+
+    # growth inside a capture is refused
+    with pytest.raises(RuntimeError, match="cannot grow during a graph capture"):
+        g0 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g0):
+            run_small()
+    torch.cuda.synchronize()
+    run_small()                                   # eager warm-up sizes the workspace (1 MiB minimum)
+    torch.cuda.synchronize()
+    ws_first = pa.reserve_decode_workspace(gpu, 1)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run_small()
+    torch.cuda.synchronize()
+    # a larger launch on the same device: more partials than the first workspace holds
+    large = cases.make_case(62, [4000] * 24, 24 * 250 + 8)
+    dl = cases.to_device(large, gpu)
+    big_out = pa.paged_decode(dl["q"], dl["k_cache"], dl["v_cache"], dl["block_tables"], dl["context_lens"],
+                              dl["scale"], partition_size=64)
+    torch.cuda.synchronize()
+    ws_second = pa.reserve_decode_workspace(gpu, 1)
+    assert ws_second.numel() > ws_first.numel() and ws_second.data_ptr() != ws_first.data_ptr()
+    check(big_out.cpu(), oracle_decode(large), "fp16")
+    # fill fresh allocations with garbage: had the first workspace been freed, this would land in it
+    junk = [torch.full((1 << 20,), float("nan"), device=gpu) for _ in range(4)]
+    for _ in range(3):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        check(out.cpu(), want, "fp16")
+        pa.paged_decode(dl["q"], dl["k_cache"], dl["v_cache"], dl["block_tables"], dl["context_lens"],
+                        dl["scale"], partition_size=64)
+        torch.cuda.synchronize()
+    del junk

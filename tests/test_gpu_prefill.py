@@ -39,11 +39,11 @@ def oracle_prefill(c, upcast=False):
                                 c["scale"], c["k_scale"], c["v_scale"], c["cache_dtype"])
 
 
-def gpu_prefill(pa, c, gpu):
+def gpu_prefill(pa, c, gpu, waves=0):
     d = cases.to_device(c, gpu)
     out = pa.paged_prefill(d["q"], d["k_cache"], d["v_cache"], d["cu_q"], d["cu_k"], c["max_q"],
                            c["scale"], block_tables=d["block_tables"], k_scale=d["k_scale"],
-                           v_scale=d["v_scale"])
+                           v_scale=d["v_scale"], waves=waves)
     torch.cuda.synchronize()
     return out.cpu()
 
@@ -57,11 +57,9 @@ def check(got, want, kind="fp16"):
 
 
 @pytest.fixture(params=[4, 8])
-def waves(request, lib):
-    """Force the 4-wave or the 8-wave workgroup shape of the prefill kernel; automatic afterwards."""
-    assert lib.pa_set_prefill_waves(request.param) == 0
-    yield request.param
-    assert lib.pa_set_prefill_waves(0) == 0
+def waves(request):
+    """The 4-wave and the 8-wave workgroup shape of the prefill kernel, forced per call."""
+    return request.param
 
 
 def test_config5a_chunked_prefill_bf16_q_fp16_kv(pa, gpu):
@@ -76,19 +74,19 @@ def test_ragged_chunks(pa, gpu, cache, waves):
     cached = [0, 5, 64, 100, 0, 333, 17]
     new = [1, 63, 64, 65, 200, 7, 130]
     c = make_prefill(60, cached, new, 96, cache=cache)
-    check(gpu_prefill(pa, c, gpu), oracle_prefill(c, upcast=True), "fp8" if cache != "fp16" else "fp16")
+    check(gpu_prefill(pa, c, gpu, waves), oracle_prefill(c, upcast=True), "fp8" if cache != "fp16" else "fp16")
 
 
 @pytest.mark.parametrize("hq,hkv,d", [(16, 8, 128), (8, 8, 128), (16, 4, 128), (8, 2, 64), (4, 4, 64)])
 def test_head_shapes(pa, gpu, hq, hkv, d, waves):
     c = make_prefill(61 + hq + d, [40, 0, 129], [70, 150, 3], 48, num_heads=hq, num_kv_heads=hkv, head_dim=d)
-    check(gpu_prefill(pa, c, gpu), oracle_prefill(c, upcast=True))
+    check(gpu_prefill(pa, c, gpu, waves), oracle_prefill(c, upcast=True))
 
 
 @pytest.mark.parametrize("bs", [8, 32])
 def test_block_sizes(pa, gpu, bs, waves):
     c = make_prefill(62, [bs * 3 + 1, 0], [100, 77], 64, block_size=bs)
-    check(gpu_prefill(pa, c, gpu), oracle_prefill(c, upcast=True))
+    check(gpu_prefill(pa, c, gpu, waves), oracle_prefill(c, upcast=True))
 
 
 def test_fp32_query(pa, gpu):
@@ -165,10 +163,12 @@ def test_module_forward_prefill_then_decode(pa, gpu):
     assert torch.equal(d["k_cache"].cpu().view(torch.int16), c["k_cache"].view(torch.int16))
 
 
-def test_waves_tunable_rejects_other_values(lib, gpu):
-    assert lib.pa_set_prefill_waves(6) != 0
-    assert b"pa_set_prefill_waves" in lib.pa_last_error()
-    assert lib.pa_set_prefill_waves(0) == 0
+def test_waves_argument_rejects_other_values(lib, gpu):
+    t = torch.zeros(64, dtype=torch.float16, device=gpu)
+    p = t.data_ptr()
+    assert lib.pa_prefill(p, 0, 2048, p, p, None, None, 0, p, 4, p, p, p, 2048, 1, 8, 16, 8, 128, 16, 4, 1.0,
+                          6, None) == -1
+    assert b"waves_per_workgroup" in lib.pa_last_error()
 
 
 def test_c_abi_argument_errors(lib, gpu):
@@ -176,7 +176,7 @@ def test_c_abi_argument_errors(lib, gpu):
     p = t.data_ptr()
     def call(d=128, hq=16, hkv=8, kvd=0, bt=p, bs=16, scale=1.0):
         return lib.pa_prefill(p, 0, hq * d, p, p, None, None, kvd, bt, 4, p, p, p, hq * d, 1, 8, hq, hkv,
-                              d, bs, 4, scale, None)
+                              d, bs, 4, scale, 0, None)
     assert call(d=96) == -2
     assert call(hq=15) == -1
     assert call(kvd=3) == -1
