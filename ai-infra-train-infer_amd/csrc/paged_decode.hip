@@ -8,6 +8,8 @@
 
 #include <stdio.h>
 
+#include <mutex>
+
 namespace pa {
 
 // out = sum_p w_p out_p / sum_p w_p, w_p = sum_p * exp(max_p - max); one workgroup per
@@ -99,6 +101,37 @@ static int ilog2_exact(int64_t v) {
   int l = 0;
   while ((int64_t(1) << l) < v) ++l;
   return l;
+}
+
+// ---- scratch of the entry point that allocates nothing ------------------------------------------
+// Partition partials of pa_decode_noalloc.  The array's name is only a host-side handle; the
+// device address is asked once per device and kept.
+constexpr int64_t kNoAllocScratchBytes = PA_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static void* g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+static int scratch_for_current_device(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(PA_ERR_LAUNCH, "pa_decode_noalloc: cannot tell the current device");
+  void* ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!ptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ptr = g_scratch_ptr[dev];
+    if (!ptr) {
+      const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !ptr) {
+        char msg[160];
+        snprintf(msg, sizeof(msg), "pa_decode_noalloc: hipGetSymbolAddress failed: HIP error %d (%s)",
+                 (int)e, hipGetErrorString(e));
+        return fail(PA_ERR_LAUNCH, msg);
+      }
+      __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+    }
+  }
+  *out = ptr;
+  return PA_OK;
 }
 
 // Shared argument checking + launch of the attention pass; `merge` adds the reduction.
@@ -283,6 +316,41 @@ extern "C" int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, con
                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
                      num_blocks, scale, partition_size, max_partitions, workspace, workspace_bytes,
                      waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, true, stream);
+}
+
+extern "C" int pa_decode_noalloc(const void* q, int q_dtype, int64_t q_token_stride,
+                                 const void* k_cache, const void* v_cache, const float* k_scale,
+                                 const float* v_scale, int kv_dtype, const int32_t* block_tables,
+                                 int64_t bt_stride, int64_t table_width, const int32_t* context_lens,
+                                 void* out, int64_t out_token_stride, int64_t batch,
+                                 int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                 int64_t block_size, int64_t num_blocks, float scale,
+                                 int64_t partition_size, int64_t max_partitions,
+                                 int waves_per_workgroup, int kv_heads_per_wave, int q_heads_per_wave,
+                         void* stream) {
+  void* ws = nullptr;
+  if (max_partitions > 1) {
+    if (batch < 0 || num_q_heads <= 0 || head_dim <= 0)
+      return fail(PA_ERR_BAD_ARG, "pa_decode_noalloc: negative or zero size");
+    const int64_t need = ws_bytes(batch, num_q_heads, head_dim, max_partitions);
+    if (need > kNoAllocScratchBytes) {
+      char msg[200];
+      snprintf(msg, sizeof(msg),
+               "pa_decode_noalloc: partials of this launch need %lld bytes, the built-in scratch holds %lld "
+               "(use pa_decode with a caller-owned workspace)",
+               (long long)need, (long long)kNoAllocScratchBytes);
+      return fail(PA_ERR_WORKSPACE, msg);
+    }
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != PA_OK) return rc;
+  }
+  // Every partial the merge reads is written by this launch's own attention pass, so nothing
+  // left in the array by an earlier call needs clearing.
+  return decode_impl("pa_decode_noalloc", q, q_dtype, q_token_stride, k_cache, v_cache, k_scale,
+                     v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, out,
+                     out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
+                     num_blocks, scale, partition_size, max_partitions, ws,
+                     ws ? kNoAllocScratchBytes : 0, waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, true, stream);
 }
 
 extern "C" int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride,

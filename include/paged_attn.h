@@ -148,6 +148,30 @@ int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, const void* k_
               int kv_heads_per_wave, int q_heads_per_wave, void* stream);
 
 /*
+ * pa_decode for callers that cannot allocate device memory or hand over a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the partition
+ * partials go to an array of PA_NOALLOC_SCRATCH_BYTES that is part of the library's device image,
+ * one copy per GPU, held until the process ends.  Same arguments and same result, bit for bit,
+ * as pa_decode without `workspace` / `workspace_bytes`; the call allocates and frees nothing.
+ * A launch whose partials need more than the array holds (pa_workspace_bytes(batch, num_q_heads,
+ * head_dim, max_partitions) > PA_NOALLOC_SCRATCH_BYTES) is refused with PA_ERR_WORKSPACE.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it and must be serialised by the caller; nothing an earlier
+ * call left in it is ever read.
+ * No counterpart in the reference (it allocates its partials as fresh tensors per call,
+ * src/inference/attention.py:456-470).
+ */
+#define PA_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int pa_decode_noalloc(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+                      const void* v_cache, const float* k_scale, const float* v_scale, int kv_dtype,
+                      const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
+                      const int32_t* context_lens, void* out, int64_t out_token_stride,
+                      int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                      int64_t block_size, int64_t num_blocks, float scale, int64_t partition_size,
+                      int64_t max_partitions, int waves_per_workgroup, int kv_heads_per_wave,
+                      int q_heads_per_wave, void* stream);
+
+/*
  * First half of the partitioned decode only: fills `workspace` and does not merge.
  * Replaces: the loop over _compute_partition_attention
  *           (src/inference/attention.py:462-470, 519-589).

@@ -47,3 +47,10 @@ def test_host_only_calls(lib):
     assert lib.pa_kv_store(None, None, 0, 0, None, None, None, 4, 1024, 2, 64, None) == -1
     assert lib.pa_decode(None, 0, 0, None, None, None, None, 0, None, 0, 0, None, None, 0, 1, 16, 8,
                          128, 16, 4, 1.0, 0, 1, None, 0, 0, 0, 0, None) == -1
+    assert lib.pa_decode_noalloc(None, 0, 0, None, None, None, None, 0, None, 0, 0, None, None, 0, 1, 16, 8,
+                                 128, 16, 4, 1.0, 0, 1, 0, 0, 0, None) == -1
+    # partials beyond the built-in scratch are refused before anything touches a GPU
+    assert lib.pa_workspace_bytes(4096, 16, 128, 64) > 16 * 1024 * 1024
+    assert lib.pa_decode_noalloc(None, 0, 0, None, None, None, None, 0, None, 0, 0, None, None, 0, 4096, 16, 8,
+                                 128, 16, 4, 1.0, 512, 64, 0, 0, 0, None) == -4
+    assert b"scratch" in lib.pa_last_error()
