@@ -43,6 +43,9 @@ SIGNATURES = {
     "pa_decode_partials": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
                                   _int, _int, _int, _ptr]),
+    "pa_decode_load_probe": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
+                                    _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr, _i64,
+                                    _int, _int, _int, _ptr]),
     "pa_merge": (_int, [_ptr, _i64, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_prefill": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr,
                           _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]),

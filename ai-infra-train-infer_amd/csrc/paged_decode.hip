@@ -134,6 +134,8 @@ static int scratch_for_current_device(void** out) {
   return PA_OK;
 }
 
+enum { kDecodeFull = 0, kDecodePartials = 1, kDecodeProbe = 2 };
+
 // Shared argument checking + launch of the attention pass; `merge` adds the reduction.
 static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_token_stride,
                        const void* k_cache, const void* v_cache, const float* k_scale,
@@ -143,8 +145,9 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
                        int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
                        int64_t num_blocks, float scale, int64_t partition_size,
                        int64_t max_partitions, void* workspace, int64_t workspace_bytes,
-                       int waves, int kv_heads_per_wave, int q_heads_per_wave, bool merge,
+                       int waves, int kv_heads_per_wave, int q_heads_per_wave, int mode,
                        void* stream) {
+  const bool merge = mode == kDecodeFull;
   char msg[256];
 #define PA_FAIL(code, text)                         \
   do {                                              \
@@ -171,6 +174,8 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   }
   if (kv == KV_FP8 && (!k_scale || !v_scale))
     PA_FAIL(PA_ERR_BAD_ARG, "fp8 cache needs k_scale and v_scale");
+  if (kv == KV_FP8 && (!aligned16(k_scale) || !aligned16(v_scale)))
+    PA_FAIL(PA_ERR_BAD_ARG, "k_scale and v_scale must be 16-byte aligned");
   if (head_dim != 64 && head_dim != 128) PA_FAIL(PA_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
   if (num_q_heads % num_kv_heads != 0)
     PA_FAIL(PA_ERR_BAD_ARG, "num_q_heads must be a multiple of num_kv_heads");
@@ -273,7 +278,14 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   }
 
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)((num_kv_heads / s.hpw) * slices), (unsigned)max_partitions, (unsigned)batch);
+  p.inner = (int)(num_kv_heads / s.hpw) * slices;
+  p.probe = mode == kDecodeProbe ? 1 : 0;
+  const int64_t wgs = batch * max_partitions * p.inner;
+  if (wgs > 0x7fffffff) {
+    snprintf(msg, sizeof(msg), "%s: too many workgroups for one launch", who);
+    return fail(PA_ERR_UNSUPPORTED, msg);
+  }
+  dim3 grid((unsigned)wgs);
   int rc;
   switch (kv) {
     case KV_F16: rc = launch_decode_f16(p, grid, s, st); break;
@@ -315,7 +327,7 @@ extern "C" int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, con
                      kv_dtype, block_tables, bt_stride, table_width, context_lens, out,
                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
                      num_blocks, scale, partition_size, max_partitions, workspace, workspace_bytes,
-                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, true, stream);
+                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodeFull, stream);
 }
 
 extern "C" int pa_decode_noalloc(const void* q, int q_dtype, int64_t q_token_stride,
@@ -350,7 +362,7 @@ extern "C" int pa_decode_noalloc(const void* q, int q_dtype, int64_t q_token_str
                      v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, out,
                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
                      num_blocks, scale, partition_size, max_partitions, ws,
-                     ws ? kNoAllocScratchBytes : 0, waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, true, stream);
+                     ws ? kNoAllocScratchBytes : 0, waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodeFull, stream);
 }
 
 extern "C" int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride,
@@ -366,7 +378,7 @@ extern "C" int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_st
                      v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, nullptr,
                      0, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale,
                      partition_size, max_partitions, workspace, workspace_bytes,
-                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, false, stream);
+                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodePartials, stream);
 }
 
 extern "C" int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* context_lens,
@@ -389,6 +401,22 @@ extern "C" int pa_merge(const void* workspace, int64_t workspace_bytes, const in
                      context_lens, out, out_dtype, out_token_stride, (int)num_q_heads,
                      (int)head_dim, (int)partition_size, (int)max_partitions);
   return check_launch("pa_merge");
+}
+
+extern "C" int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride,
+                                    const void* k_cache, const void* v_cache, const float* k_scale,
+                                    const float* v_scale, int kv_dtype, const int32_t* block_tables,
+                                    int64_t bt_stride, int64_t table_width, const int32_t* context_lens,
+                                    int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    int64_t partition_size, int64_t max_partitions, void* workspace,
+                                    int64_t workspace_bytes, int waves_per_workgroup,
+                                    int kv_heads_per_wave, int q_heads_per_wave, void* stream) {
+  return decode_impl("pa_decode_load_probe", q, q_dtype, q_token_stride, k_cache, v_cache, k_scale,
+                     v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, nullptr,
+                     0, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, 1.0f,
+                     partition_size, max_partitions, workspace, workspace_bytes,
+                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodeProbe, stream);
 }
 
 extern "C" int pa_check_tables(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,

@@ -63,6 +63,8 @@ struct DecodeParams {
   int partition_size;
   int max_partitions;
   int direct_out;
+  int inner;        // workgroups per (batch row, partition): KV head groups x slices of the query group
+  int probe;        // 1: loads only, the arithmetic replaced by a checksum (pa_decode_load_probe)
   float scale_log2e;
 };
 
@@ -147,6 +149,15 @@ __device__ __forceinline__ void unpack(const uint32_t (&w)[WPT], float (&x)[EPL]
   }
 }
 
+// Which token a lane holds in row load r of a tile.  16-bit caches: token r * RPL + tr (the 8 / HPW
+// tokens of a row load are consecutive, so one table entry serves the whole load).  fp8 caches:
+// token tr * RL + r - a lane's RL = 4 tokens are consecutive, so their per-token scales are one
+// 16-byte load per lane and tile for K and one for V instead of a 4-byte load per row load (10
+// vector memory instructions per fp8 tile instead of 16; the data loads are the same 128-byte
+// rows either way).
+template <int KV>
+constexpr bool kLaneMajorTokens = (KV == KV_FP8);
+
 template <int KV, int D, int HPW>
 struct Tile {
   using G = Geo<KV, D, HPW>;
@@ -191,17 +202,19 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   const int j = lane & 7;         // position inside the row
   const int hs = g % HPW;         // which of the wave's KV heads this row group reads
   const int tr = g / HPW;         // token inside a row load
-  // blockIdx.x (fastest) walks the KV head groups first, so the workgroups that share a token
-  // row are dispatched together and land on different XCDs (each L2 fetches only its own heads'
-  // bytes), and then - only when one workgroup cannot hold a KV head's whole query group - the
-  // slices of the query group: with 8 KV head groups those land on the same XCD as their
-  // siblings and share its L2.
-  const int b = blockIdx.z;
-  const int part = blockIdx.y;
+  // Workgroups go to the 8 XCDs round robin by their index.  blockIdx.x walks the KV head groups
+  // first, so the workgroups that share a token row are dispatched together and land on
+  // different XCDs: each L2 fetches only its own heads' bytes (putting them on one XCD instead
+  // measured 3% slower).  Then - only when one workgroup cannot hold a KV head's whole query
+  // group - the slices of the query group.
+  const int in = blockIdx.x % p.inner;
+  const int u = blockIdx.x / p.inner;
+  const int part = u % p.max_partitions;
+  const int b = u / p.max_partitions;
   const int gq = p.num_q_heads / p.num_kv_heads;
   const int kv_groups = p.num_kv_heads / HPW;
-  const int kvg = blockIdx.x % kv_groups;
-  const int sub = blockIdx.x / kv_groups;
+  const int kvg = in % kv_groups;
+  const int sub = in / kv_groups;
   const int h0 = kvg * HPW * gq + sub * (GC * QS);    // first query head of the workgroup
   const int kvh = kvg * HPW + hs;                     // this lane's KV head
   const int hl0 = (hs + qgrp) * GC;                   // this lane's first query head, relative to h0
@@ -256,7 +269,15 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   const int bs_mask = (1 << p.bs_log2) - 1;
   const uint32_t token_bytes = (uint32_t)(p.num_kv_heads * D * G::ES);
   const uint32_t block_bytes = token_bytes << p.bs_log2;
-  const uint32_t lane_off = (uint32_t)((tr * p.num_kv_heads + kvh) * D * G::ES + j * G::LB);
+  constexpr bool LM = kLaneMajorTokens<KV>;
+  // lane-major tiles: which of the tile's RL table entries (one per RPL tokens) covers this
+  // lane's tokens tr * RL ... tr * RL + RL - 1
+  int id_mask[RL];
+#pragma unroll
+  for (int r = 0; r < RL; ++r) id_mask[r] = (LM && (tr * RL) / RPL == r) ? -1 : 0;
+  // byte offset of the lane's piece from the first token of its row load (row-major tiles: tr
+  // tokens further on) or of its own token group (lane-major tiles)
+  const uint32_t lane_off = (uint32_t)(((LM ? 0 : tr) * p.num_kv_heads + kvh) * D * G::ES + j * G::LB);
   const int32_t* bt_row = p.block_tables + b * p.bt_stride;
   // never index past the table row, even if a context length is larger than the row holds
   const int last_blk = min((end - 1) >> p.bs_log2, max(p.table_width - 1, 0));
@@ -275,36 +296,73 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
   // start the K/V (and scale) loads of a tile; ids are clamped to the pool so that a corrupt
   // table can never fault
   auto issue = [&](TileT& t, int tile, const int (&ids)[RL]) {
+    if constexpr (LM) {
+      static_assert(!LM || RL == 4, "lane-major tiles load four scales at once");
+      // the table entry of this lane's four tokens: one of the tile's RL wave-uniform entries
+      // (picked with per-lane bit masks: written as selects over the array, the compiler turns
+      // the chain into an indexed read of a copy of `ids` in scratch memory)
+      int id = 0;
 #pragma unroll
-    for (int r = 0; r < RL; ++r) {
-      const int tok = begin + tile * TILE + r * RPL;
-      const uint32_t phys = (uint32_t)min(max(ids[r], 0), p.num_blocks - 1);
-      const uint32_t off = (uint32_t)(tok & bs_mask);
-      const uint64_t base = (uint64_t)phys * block_bytes + off * token_bytes;
+      for (int r = 0; r < RL; ++r) id |= ids[r] & id_mask[r];
+      const uint32_t phys = (uint32_t)min(max(id, 0), p.num_blocks - 1);
+      const uint32_t off = (uint32_t)((begin + tile * TILE + tr * RL) & bs_mask);
+      const uint64_t base = (uint64_t)phys * block_bytes + off * token_bytes + lane_off;
       const uint8_t* kp = p.k_cache + base;
       const uint8_t* vp = p.v_cache + base;
 #pragma unroll
-      for (int c = 0; c < G::NLD; ++c) {
-        load_words<G::LB>(kp + (lane_off + c * G::LPR * G::LB), &t.k[r][c * (G::LB / 4)]);
-        load_words<G::LB>(vp + (lane_off + c * G::LPR * G::LB), &t.v[r][c * (G::LB / 4)]);
+      for (int r = 0; r < RL; ++r) {
+#pragma unroll
+        for (int c = 0; c < G::NLD; ++c) {
+          load_words<G::LB>(kp + (r * token_bytes + c * G::LPR * G::LB), &t.k[r][c * (G::LB / 4)]);
+          load_words<G::LB>(vp + (r * token_bytes + c * G::LPR * G::LB), &t.v[r][c * (G::LB / 4)]);
+        }
       }
-      if constexpr (KV == KV_FP8) {
-        const uint64_t slot = ((uint64_t)phys << p.bs_log2) + off;
-        t.ks[r] = p.k_scale[slot + tr];
-        t.vs[r] = p.v_scale[slot + tr];
+      const uint64_t slot = ((uint64_t)phys << p.bs_log2) + off;
+      const float4 k4 = *(const float4*)(p.k_scale + slot);
+      const float4 v4 = *(const float4*)(p.v_scale + slot);
+      t.ks[0] = k4.x; t.ks[1] = k4.y; t.ks[2] = k4.z; t.ks[3] = k4.w;
+      t.vs[0] = v4.x; t.vs[1] = v4.y; t.vs[2] = v4.z; t.vs[3] = v4.w;
+    } else {
+#pragma unroll
+      for (int r = 0; r < RL; ++r) {
+        const int tok = begin + tile * TILE + r * RPL;
+        const uint32_t phys = (uint32_t)min(max(ids[r], 0), p.num_blocks - 1);
+        const uint32_t off = (uint32_t)(tok & bs_mask);
+        const uint64_t base = (uint64_t)phys * block_bytes + off * token_bytes;
+        const uint8_t* kp = p.k_cache + base;
+        const uint8_t* vp = p.v_cache + base;
+#pragma unroll
+        for (int c = 0; c < G::NLD; ++c) {
+          load_words<G::LB>(kp + (lane_off + c * G::LPR * G::LB), &t.k[r][c * (G::LB / 4)]);
+          load_words<G::LB>(vp + (lane_off + c * G::LPR * G::LB), &t.v[r][c * (G::LB / 4)]);
+        }
       }
     }
   };
 
   auto consume = [&](TileT& t, int tile, auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
+    if (p.probe) {
+      // timing aid: every loaded word is used, none of the attention arithmetic is done
+      uint32_t x = 0;
+#pragma unroll
+      for (int r = 0; r < RL; ++r) {
+#pragma unroll
+        for (int i = 0; i < G::WPT; ++i) x ^= t.k[r][i] ^ t.v[r][i];
+        if constexpr (KV == KV_FP8) x ^= __float_as_uint(t.ks[r]) ^ __float_as_uint(t.vs[r]);
+      }
+      acc[0][0] += __uint_as_float(x & 0x3fffffffu);
+      l[0] = 1.0f;
+      m[0] = 0.0f;
+      return;
+    }
     float s[RL][GC];
     bool valid[RL];
 #pragma unroll
     for (int r = 0; r < RL; ++r) valid[r] = true;
 #pragma unroll
     for (int r = 0; r < RL; ++r) {
-      if constexpr (MASKED) valid[r] = (begin + tile * TILE + r * RPL + tr) < end;
+      if constexpr (MASKED) valid[r] = (begin + tile * TILE + (LM ? tr * RL + r : r * RPL + tr)) < end;
       float kf[EPL];
       unpack<KV, G::WPT, EPL>(t.k[r], kf);
       float inv_ks = 1.0f;

@@ -593,6 +593,22 @@ def main():
                             w["context_lens"], scale, w["k_scale"], w["v_scale"], out=w["out"])
 
         fns[kind] = step
+        # the same launch with the arithmetic taken out: what the memory system needs for this
+        # access pattern alone
+        pbytes = lib.pa_workspace_bytes(B, HQ, D, parts)
+        w["probe_ws"] = torch.empty(max(pbytes, 256), dtype=torch.uint8, device=dev)
+
+        def probe(w=w, fp8=fp8, psize=psize, parts=parts, hpw=hpw):
+            rc = lib.pa_decode_load_probe(
+                w["q"].data_ptr(), 0, HQ * D, w["k_cache"].data_ptr(), w["v_cache"].data_ptr(),
+                w["k_scale"].data_ptr() if fp8 else None, w["v_scale"].data_ptr() if fp8 else None,
+                pa._native.DTYPE_FP8_E4M3 if fp8 else pa._native.DTYPE_F16, w["block_tables"].data_ptr(),
+                w["block_tables"].stride(0), w["block_tables"].shape[1], w["context_lens"].data_ptr(),
+                B, HQ, HKV, D, BS, w["num_blocks"], max(psize, 16), parts, w["probe_ws"].data_ptr(),
+                w["probe_ws"].numel(), 0, hpw, 0, stream)
+            assert rc == 0, lib.pa_last_error()
+
+        fns[kind + "_probe"] = probe
         if parts > 1:
             # dominant kernel alone: the attention pass without the merge (a single-pass launch IS
             # that one kernel, so its operator timing is used as it stands)
@@ -621,7 +637,7 @@ def main():
         k_us = t.get(kind + "_kernel", us)
         assert med(k_us) <= med(us) * 1.02, "the attention pass alone cannot take longer than the call that contains it"
         nbytes_alg = algorithmic_bytes(B, CTX, HQ, HKV, D, BS, kind == "fp8")
-        results[kind] = dict(us=us, kernel_us=k_us, bytes=nbytes_alg,
+        results[kind] = dict(us=us, kernel_us=k_us, bytes=nbytes_alg, probe_us=t[kind + "_probe"],
                              gbps=nbytes_alg / med(us) / 1e3, kernel_gbps=nbytes_alg / min(med(k_us), med(us)) / 1e3,
                              partition_size=shape[kind][0], partitions=shape[kind][1], kv_heads_per_wave=shape[kind][2])
     if not args.no_cpu_baseline:
@@ -694,6 +710,13 @@ def main():
             "fp8_kernel": {"achieved": round(f8["kernel_gbps"], 1), "frac": round(f8["kernel_gbps"] / HBM_PEAK_GBPS, 4),
                            "algorithmic_bytes": f8["bytes"],
                            "traffic": measured_traffic("traffic_bytes_fp8") if (B, CTX) == (64, 4096) else None},
+            "loads_only": {
+                "what": "pa_decode_load_probe: the same launches with every load issued and consumed but no "
+                        "attention arithmetic, i.e. the rate the memory system gives this access pattern",
+                "fp16_us": spread(f16["probe_us"]), "fp16_gbps": round(f16["bytes"] / med(f16["probe_us"]) / 1e3, 1),
+                "fp8_us": spread(f8["probe_us"]), "fp8_gbps": round(f8["bytes"] / med(f8["probe_us"]) / 1e3, 1),
+                "fp16_kernel_vs_loads_only": round(med(f16["probe_us"]) / min(med(f16["kernel_us"]), med(f16["us"])), 3),
+                "fp8_kernel_vs_loads_only": round(med(f8["probe_us"]) / min(med(f8["kernel_us"]), med(f8["us"])), 3)},
         },
     }
     line["other_configs"] = other_decode_configs(pa, torch, dev, launches)

@@ -191,6 +191,25 @@ int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const
                        void* stream);
 
 /*
+ * Timing aid: the launch of pa_decode_partials with the attention arithmetic taken out.  Every
+ * K, V, scale and table load of the real launch is issued from the same lanes in the same order
+ * and every loaded word is consumed (a checksum lands in `workspace`), but no dot product,
+ * exponential or accumulation is done.  Its duration is what the memory system needs for this
+ * access pattern alone - the ceiling the decode kernel is measured against besides the nominal
+ * HBM rate.  Arguments as pa_decode_partials (no scale factor); the workspace contents are
+ * meaningless afterwards.  No counterpart in the reference.
+ */
+int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+                         const void* v_cache, const float* k_scale, const float* v_scale,
+                         int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
+                         int64_t table_width, const int32_t* context_lens, int64_t batch,
+                         int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                         int64_t block_size, int64_t num_blocks, int64_t partition_size,
+                         int64_t max_partitions, void* workspace, int64_t workspace_bytes,
+                         int waves_per_workgroup, int kv_heads_per_wave, int q_heads_per_wave,
+                         void* stream);
+
+/*
  * Merge reduction over partitions.
  * Replaces: PartitionedPagedAttention._merge_partitions (src/inference/attention.py:591-626).
  * out = sum_p w_p * out_p / sum_p w_p with w_p = sum_p * exp(max_p - max_all), over the
