@@ -263,6 +263,10 @@ class KVCacheManager:
         """Block table for a new sequence of num_initial_tokens tokens.  shared_block_ids are full
         blocks that already hold the first len(shared) * block_size tokens; they gain an owner
         instead of being allocated.  Raises RuntimeError (after rolling back) when out of blocks."""
+        if seq_id in self._seq_tables:
+            # replacing the table would leak every block the sequence already owns
+            raise RuntimeError("allocate_for_sequence: seq %s already has a block table "
+                               "(free_sequence it first)" % (seq_id,))
         table = BlockTable(self._block_size)
         shared = list(shared_block_ids or [])
         needed = (num_initial_tokens + self._block_size - 1) // self._block_size
@@ -295,6 +299,8 @@ class KVCacheManager:
         parent = self._seq_tables.get(parent_id)
         if parent is None:
             raise RuntimeError("fork_sequence: unknown parent %s" % (parent_id,))
+        if child_id in self._seq_tables:
+            raise RuntimeError("fork_sequence: seq %s already has a block table" % (child_id,))
         table = BlockTable(self._block_size)
         for block in parent.blocks:
             table.append_block(self._pool.share(block))
@@ -342,11 +348,29 @@ class KVCacheManager:
     def pending_copies(self) -> List[Tuple[int, int]]:
         return list(self._pending_copies)
 
+    @staticmethod
+    def _ordered_batches(pairs: List[Tuple[int, int]]) -> List[List[Tuple[int, int]]]:
+        """Cut the queue, in order, into batches in which no block is written by one pair and read
+        or written by another: the pairs of one launch run concurrently, launches run in order.
+        A queue can chain when the pool is nearly full: block X is queued as the source of (X, Y),
+        its last owner frees it, and the next copy-on-write is handed X as its destination."""
+        batches, current, reads, writes = [], [], set(), set()
+        for src, dst in pairs:
+            if src in writes or dst in writes or dst in reads:
+                batches.append(current)
+                current, reads, writes = [], set(), set()
+            current.append((src, dst))
+            reads.add(src)
+            writes.add(dst)
+        if current:
+            batches.append(current)
+        return batches
+
     def apply_copies(self):
-        """Run the queued copy-on-write copies on the current stream."""
-        if self._pending_copies:
-            self._pool.copy_blocks(self._pending_copies)
-            self._pending_copies = []
+        """Run the queued copy-on-write copies on the current stream, in queue order."""
+        pending, self._pending_copies = self._pending_copies, []
+        for batch in self._ordered_batches(pending):
+            self._pool.copy_blocks(batch)
 
     def free_sequence(self, seq_id):
         table = self._seq_tables.pop(seq_id, None)

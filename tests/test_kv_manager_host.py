@@ -177,3 +177,78 @@ def test_copy_blocks_on_cpu_pool_fails_loudly():
     with pytest.raises(RuntimeError, match="no CPU path"):
         p.copy_blocks([(0, 1)])
     p.copy_blocks([])            # nothing to do is fine anywhere
+
+
+def test_duplicate_sequence_ids_are_refused():
+    p = pool(8)
+    m = pa.KVCacheManager(p, BS)
+    m.allocate_for_sequence("a", BS + 1)
+    with pytest.raises(RuntimeError, match="already has a block table"):
+        m.allocate_for_sequence("a", 1)
+    with pytest.raises(RuntimeError, match="already has a block table"):
+        m.fork_sequence("a", "a")
+    assert p.num_used_blocks == 2                   # nothing leaked, nothing replaced
+    m.free_sequence("a")
+    m.allocate_for_sequence("a", 1)
+    assert p.num_used_blocks == 1
+
+
+def test_chained_copies_are_cut_into_ordered_launches():
+    cut = pa.KVCacheManager._ordered_batches
+    assert cut([]) == []
+    assert cut([(1, 2), (3, 4), (1, 5)]) == [[(1, 2), (3, 4), (1, 5)]]          # shared sources are fine
+    assert cut([(1, 2), (2, 3)]) == [[(1, 2)], [(2, 3)]]                          # reads what the first writes
+    assert cut([(1, 2), (7, 1)]) == [[(1, 2)], [(7, 1)]]                          # overwrites what the first reads
+    assert cut([(1, 2), (3, 2), (4, 5)]) == [[(1, 2)], [(3, 2), (4, 5)]]          # same destination twice
+
+
+def test_a_freed_source_reused_as_destination_is_copied_in_order():
+    """Nearly full pool: block 0 is queued as a copy's source, its last owner leaves, and a later
+    copy-on-write is handed block 0 as its destination.  The launches keep the queue's order."""
+    p = pool(4)
+    m = pa.KVCacheManager(p, BS)
+    m.allocate_for_sequence("a", 2)                 # block 0, half full
+    m.fork_sequence("a", "b")
+    assert m.append_token("b")                      # b moves to a copy: (0 -> 1)
+    m.free_sequence("a")                            # block 0 loses its last owner: free again
+    m.allocate_for_sequence("c", 2)                 # block 2
+    m.fork_sequence("c", "d")
+    assert m.append_token("d")                      # (2 -> 3)
+    m.fork_sequence("c", "g")
+    assert m.append_token("g")                      # the only free block is 0: (2 -> 0)
+    assert m.pending_copies == [(0, 1), (2, 3), (2, 0)]
+    launched = []
+    p.copy_blocks = lambda pairs: launched.append(list(pairs))
+    m.apply_copies()
+    assert launched == [[(0, 1), (2, 3)], [(2, 0)]] and m.pending_copies == []
+
+
+def test_prefix_hash_is_the_documented_xxh64_chain():
+    """compute_block_hash == xxh64 over (previous hash as 8 LE bytes) + (token ids as 4-byte LE
+    words), fed here one word at a time through the streaming interface."""
+    import xxhash
+    c = pa.PrefixCache(block_size=BS)
+    toks, prev = [7, 0, 2 ** 31 + 5, 151935], 0x0123456789ABCDEF
+    h = xxhash.xxh64()
+    h.update(prev.to_bytes(8, "little"))
+    for t in toks:
+        h.update(t.to_bytes(4, "little"))
+    assert c.compute_block_hash(toks, prev) == h.intdigest()
+    first = xxhash.xxh64(b"\0" * 8 + b"".join(t.to_bytes(4, "little") for t in toks)).intdigest()
+    assert c.block_hashes(toks + toks) == [first, c.compute_block_hash(toks, first)]
+
+
+def test_prefix_cache_eviction_order():
+    c = pa.PrefixCache(block_size=1, max_cached_blocks=3)
+    c.insert([10], [0]); c.insert([20], [1]); c.insert([30], [2])
+    assert c.match_prefix([10]) == (1, [0])         # 10 is in use and now the most recently touched
+    c.insert([40], [3])                             # evicts the oldest idle entry: 20
+    assert c.match_prefix([20])[0] == 0 and c.size == 3
+    c.release_block(c.compute_block_hash([10]))     # 10 idle again, but still younger than 30
+    c.insert([50], [4])                             # so 30 goes
+    assert c.match_prefix([30])[0] == 0
+    assert c.match_prefix([10]) == (1, [0]) and c.match_prefix([40]) == (1, [3])
+    # everything in use: the least recently used of them is evicted all the same
+    assert c.match_prefix([50]) == (1, [4])
+    c.insert([60], [5])
+    assert c.size == 3 and c.match_prefix([10])[0] == 0 and c.get_stats()["evictions"] == 3
