@@ -9,13 +9,20 @@ from oracle import paged_attention_oracle as oracle
 
 pytestmark = pytest.mark.gpu
 
-# bf16 has no stated tolerance: its 8-bit mantissa (output and oracle arithmetic) sets 2e-2 / 1e-2
-TOL = {"fp16": dict(rtol=1e-3, atol=2e-3), "bf16": dict(rtol=2e-2, atol=1e-2),
+# bf16 (no tolerance is stated for it): the oracle is evaluated in fp32 on the bf16 inputs, and the
+# GPU result may differ from it by the 16-bit tolerance plus the one rounding of the output to
+# bf16 (2^-8 relative) - the scheme of the prefill tests.
+TOL = {"fp16": dict(rtol=1e-3, atol=2e-3), "bf16": dict(rtol=1e-3 + 2.0 ** -8, atol=2e-3),
        "fp8": dict(rtol=1e-2, atol=1e-2)}
 
 
 def oracle_decode(c):
-    return oracle.decode(c["q"], c["k_cache"], c["v_cache"], c["block_tables"], c["context_lens"],
+    q, kc, vc = c["q"], c["k_cache"], c["v_cache"]
+    if q.dtype == torch.bfloat16 or kc.dtype == torch.bfloat16:
+        q = q.float()
+        if kc.dtype != cases.FP8:
+            kc, vc = kc.float(), vc.float()
+    return oracle.decode(q, kc, vc, c["block_tables"], c["context_lens"],
                          c["scale"], c["k_scale"], c["v_scale"], c["cache_dtype"])
 
 
@@ -96,9 +103,8 @@ def test_query_dtypes_against_fp64(pa, gpu, qdt):
     assert got.dtype == qdt
     want = oracle.decode_f64(c["q"], c["k_cache"], c["v_cache"], c["block_tables"],
                              c["context_lens"], c["scale"])
-    torch.testing.assert_close(got.double(), want, rtol=1e-3 if qdt == torch.float32 else 1e-2,
-                               atol=2e-3 if qdt == torch.float32 else 1e-2)
-    check(got, oracle_decode(c), "fp16" if qdt == torch.float32 else "fp8")
+    torch.testing.assert_close(got.double(), want, **TOL["fp16" if qdt == torch.float32 else "bf16"])
+    check(got, oracle_decode(c), "fp16" if qdt == torch.float32 else "bf16")
 
 
 def test_fp32_query_is_accurate_to_fp32_level(pa, gpu):
