@@ -28,6 +28,12 @@
 //    transpose load of gfx950 (16 lanes read a 4-key x 16-dim patch and each gets the 4 keys of
 //    its own column).  The two 4-key groups a lane fetches are the keys the S^T layout gives that
 //    lane half, so no shuffle sits between the two products.
+//  * The softmax costs a lane an exp2, half a conversion, half a dot-2 add and a third of a max per
+//    score: Q is multiplied by scale * log2(e) once, on its way into fp16; the score products
+//    start from a block of registers holding minus the row's reference point, so the matrix pipe
+//    delivers exp2 arguments; probabilities are converted to fp16 in pairs and the row sum adds
+//    those pairs (v_dot2c_f32_f16 with ones), i.e. exactly what the second product multiplies;
+//    the two lane halves of a query column compare maxima with one v_permlane32_swap.
 //  * The mask is applied only on tiles that cross the diagonal or the end of the sequence.
 #include "pa_common.hpp"
 #include "pa_host.hpp"
@@ -43,6 +49,8 @@ namespace pa {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v_t __attribute__((ext_vector_type(2)));
+typedef unsigned uint2v_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 struct PrefillParams {
@@ -230,7 +238,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
         float x[8];
         load8_as_f32(p.q, base + ks * 16, decltype(dt_tag)::value, x);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qreg[ks][e] = (_Float16)x[e];
+        for (int e = 0; e < 8; ++e) qreg[ks][e] = (_Float16)(x[e] * p.scale_log2e);
       }
     };
     if (p.q_dtype == PA_DTYPE_F16) load_q(std::integral_constant<int, PA_DTYPE_F16>{});
@@ -243,8 +251,14 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[mt][i] = 0.0f;
-  float m_run = NEG_INF;  // running max of raw scores (same in both lane halves)
   float l_run = 0.0f;     // running sum of this lane half's probabilities
+  // Q carries scale * log2(e), and the first product of every score tile starts from the block
+  // neg_ref (-m_ref in all 16 registers) instead of zero: the matrix pipe hands back
+  // s * scale * log2(e) - m_ref, ready for exp2, and the softmax needs no multiply-add per score.
+  float m_ref = 0.0f;     // reference point of the exponentials (same in both lane halves)
+  float16_t neg_ref;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) neg_ref[i] = 0.0f;
 
   // keys the workgroup needs: up to the last valid row's limit
   const int last_tok = min(tok0 + BM, lq) - 1;
@@ -287,7 +301,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
   }
   auto move_chunk = [&](int c, int buf, const uint8_t* kp, const uint8_t* vp, int64_t slot) __attribute__((always_inline)) {
     if constexpr (DIRECT) {
-      const int wbase = (NT * c + (tid & ~63)) * 8;   // LDS destination = wave base + lane * 16 bytes
+      const int wbase = (NT * c + wave * 64) * 8;     // LDS destination = wave base + lane * 16 bytes
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
                                        (__attribute__((address_space(3))) void*)&lds.k[buf][wbase], 16, 0, 0);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
@@ -309,21 +323,35 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
     const int row0 = (NT * (lane % NCH) + 64 * wave) / CPR;
     return bt_row[min((t * kBN + row0) >> p.bs_log2, bt_last)];
   };
+  // wave-uniform 64-bit pointer in scalar registers: with the lane's constant 32-bit offset added
+  // the load takes the "scalar base + vector offset" form
+  auto uniform_ptr = [](const uint8_t* q) __attribute__((always_inline)) {
+    const uint64_t a = (uint64_t)(uintptr_t)q;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+  };
   auto fetch = [&](int t, int buf, int ids) __attribute__((always_inline)) {
     if (uniform_rows && (t + 1) * kBN <= lk) {
+      // straight-line code per addressing mode: the waves of a workgroup leave the barrier together
+      // and fetch the same instructions, and every taken branch costs each of them a refill
+      if (bt_row) {
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const int row0 = (NT * c + 64 * wave) / CPR;      // first row of this wave's instruction
-        const int key0 = t * kBN + row0;
-        int64_t slot0;
-        if (bt_row) {
+        for (int c = 0; c < NCH; ++c) {
+          const int key0 = t * kBN + (NT * c) / CPR + wave * (64 / CPR);   // first row of this wave's instruction
           const int phys = min(max(__builtin_amdgcn_readlane(ids, c), 0), p.num_blocks - 1);
-          slot0 = ((int64_t)phys << p.bs_log2) + (key0 & bs_mask);
-        } else {
-          slot0 = (int64_t)k0 + key0;
+          const int64_t slot0 = ((int64_t)phys << p.bs_log2) + (key0 & bs_mask);
+          const int64_t base = slot0 * token_elems * ES;
+          move_chunk(c, buf, uniform_ptr(p.k + base) + lane_part[c], uniform_ptr(p.v + base) + lane_part[c], slot0 + lane / CPR);
         }
-        const int64_t base = slot0 * token_elems * ES;
-        move_chunk(c, buf, p.k + base + lane_part[c], p.v + base + lane_part[c], slot0 + lane / CPR);
+      } else {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          const int key0 = t * kBN + (NT * c) / CPR + wave * (64 / CPR);
+          const int64_t slot0 = (int64_t)k0 + key0;
+          const int64_t base = slot0 * token_elems * ES;
+          move_chunk(c, buf, uniform_ptr(p.k + base) + lane_part[c], uniform_ptr(p.v + base) + lane_part[c], slot0 + lane / CPR);
+        }
       }
       return;
     }
@@ -390,7 +418,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+      for (int i = 0; i < 16; ++i) s[kt][i] = neg_ref[i];
     // All K fragments of the first 32-key half are requested at once and those of the second
     // half as the first are consumed, so a product never waits for a read issued just before it.
     constexpr int OFF0 = buf * kBN * D * 2, OFF1 = OFF0 + 32 * D * 2;
@@ -423,42 +451,56 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
           s[kt][i] = key <= lim ? s[kt][i] : NEG_INF;
         }
     }
-    // ---- online softmax over this lane's query column ---------------------------------------------
-    float mloc = s[0][0];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    // Lazy rescale: the running max only follows the true max when it has grown by more than
-    // 2^8 in the exponent domain, so probabilities stay <= 256 (exact enough in fp16 and fp32)
-    // and the 64-register rescale of O^T runs on the first tile and then almost never.  The
-    // final division by the row sum removes whatever reference point was used.
-    const float c = p.scale_log2e;
-    const bool grow = (mloc - m_run) * c > 8.0f;
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(grow) != 0, 0)) {
-      const float m_new = grow ? mloc : m_run;
-      // exp2(-inf) = 0 on a row's first visible tile; rows that do not move keep factor 1
-      const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * c) : 1.0f;
-      l_run *= alpha;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
-      m_run = m_new;
-    }
-    const float mc = (m_run == NEG_INF ? 0.0f : m_run) * c;
-    float psum = 0.0f;
     half8_t pb[4];
+    {
+      // ---- online softmax over this lane's query column; the scores arrive in the exponent domain,
+      // relative to m_ref ---------------------------------------------------------------------------
+      float mloc = s[0][0];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float pr = __builtin_amdgcn_exp2f(fmaf(s[kt][i], c, -mc));
-        psum += pr;
-        pb[kt * 2 + (i >> 3)][i & 7] = (_Float16)pr;
+        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kt][i]);
+      {
+        // the other 16 keys of this query column sit 32 lanes away
+        const uint2v_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mloc), __float_as_uint(mloc), false, false);
+        mloc = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
       }
-    l_run += psum;
+      // Lazy rescale: the first tile sets the reference to its maximum; later it only follows the
+      // true maximum when that has outgrown it by more than 2^8, so probabilities stay <= 256
+      // (exact enough in fp16 and fp32) and the rescale of the 64 accumulator registers, of this
+      // tile's scores and of the reference block almost never runs.  The final division by the
+      // row sum removes whatever reference point was used.  A row with no visible key yet (all
+      // scores -inf) keeps reference 0 and adds nothing.
+      const bool grow = (t == 0) ? (mloc > NEG_INF) : (mloc > 8.0f);
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(grow) != 0, 0)) {
+        const float delta = grow ? mloc : 0.0f;
+        const float alpha = (t == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);   // accumulators are zero on the first tile
+        l_run *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[kt][i] -= delta;
+        m_ref += delta;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) neg_ref[i] = -m_ref;
+      }
+      float psum = 0.0f;
+      const half2v_t one2 = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const half2v_t h = {(_Float16)__builtin_amdgcn_exp2f(s[kt][i]), (_Float16)__builtin_amdgcn_exp2f(s[kt][i + 1])};
+          psum = __builtin_amdgcn_fdot2(h, one2, psum, false);   // the row sum adds what the second product multiplies
+          pb[kt * 2 + (i >> 3)][i & 7] = h[0];
+          pb[kt * 2 + (i >> 3)][(i & 7) + 1] = h[1];
+        }
+      l_run += psum;
+    }
     // ---- O^T += V^T . P^T : four 16-key steps x MT row tiles ----------------------------------------
     // untracked reads, one 16-key step ahead of the products that use them
     half4_t lo[2][MT], hi[2][MT];
@@ -510,12 +552,13 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
   __syncthreads();
   auto step = [&](int t, auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
-    if (t + 1 < ntiles) {
+    const bool more = t + 1 < ntiles;
+    if (more) {
       fetch(t + 1, buf ^ 1, ids);      // direct loads land in the other buffer while this one is used
       if (t + 2 < ntiles) ids = load_ids(t + 2);
     }
     if (wave_has_rows && t * kBN <= wave_last) compute(t, buf_tag);
-    if (t + 1 < ntiles) commit(buf ^ 1);
+    if (more) commit(buf ^ 1);
     __syncthreads();                   // also waits for this wave's outstanding loads into LDS
   };
   for (int t = 0; t < ntiles; t += 2) {
