@@ -1,6 +1,6 @@
 """Benchmark of the paged decode attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--sections a,b,...]
 
 Workload (BASELINE.json configs[1] shape, the one the metric is quoted on): batch 64, context
 4096 per sequence, 16 query / 8 KV heads, head_dim 128, block_size 16, block tables a random
@@ -17,7 +17,8 @@ what the command line asked for; the launches actually timed are under `timing`.
 Prints ONE JSON line.  `roofline` is for the dominant kernel (the attention pass alone);
 `cpu_baseline` times the oracle (the reference's PyTorch fallback restated) on a bounded
 sample of the same workload.  `other_configs` holds the decode launches of BASELINE configs 1,
-3 and 4 (same recipe as the parity tests: seeds 1001 / 1003 / 1004).
+3 and 4 (same recipe as the parity tests: seeds 1001 / 1003 / 1004) and of 32 and 64 query heads
+over the 8 KV heads at the headline batch and context.
 """
 import argparse
 import json
@@ -258,11 +259,25 @@ def other_decode_configs(pa, torch, dev, launches):
     meta["cfg4"] = dict(workload="32 prompts x 8 samples, shared 1024-token prefix, suffix U[64,512] (seed 1004), FP16 KV",
                         kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
+    # wider GQA groups at the headline batch and context: every KV row is still read once, by the
+    # one workgroup that serves all query heads of its KV head
+    gqa = {}
+    for name, hq in (("gqa4", 32), ("gqa8", 64)):
+        w, _ = _paged_case(torch, dev, [4096] * 64, 1100 + hq, hq=hq)
+        gqa[name] = w
+        fns[name] = lambda w=w: pa.paged_decode(w["q"], w["k_cache"], w["v_cache"], w["block_tables"],
+                                                w["context_lens"], scale, out=w["out"])
+        meta[name] = dict(workload="batch 64, ctx 4096, %d q / 8 kv heads (GQA %d), FP16 KV" % (hq, hq // 8),
+                          alg_bytes=algorithmic_bytes(64, 4096, hq, HKV, D, BS, False))
+
     t = time_alternating(torch, fns, launches)
     for name, m in meta.items():
         us = med(t[name])
         rec = {"workload": m["workload"], "us": spread(t[name])}
-        if "note" in m:
+        if "alg_bytes" in m:
+            rec.update(algorithmic_bytes=m["alg_bytes"], gbps=round(m["alg_bytes"] / us / 1e3, 1),
+                       frac_of_8TBps=round(m["alg_bytes"] / us / 1e3 / HBM_PEAK_GBPS, 4))
+        elif "note" in m:
             rec["note"] = m["note"]
             rec["kv_bytes"] = m["kv_bytes"]
         elif "unique_kv_bytes" in m:
@@ -298,7 +313,7 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup):
     def step():
         pa.paged_prefill(q, kc, vc, cu_q, cu_k, NEW, D ** -0.5, block_tables=tables, out=out)
 
-    us = time_alternating(torch, {"prefill": step}, max(steps, MIN_LAUNCHES), warmup=max(warmup, 20))["prefill"]
+    us = time_alternating(torch, {"prefill": step}, steps, warmup=max(warmup, 20))["prefill"]
     ms = med(us) / 1e3
     pairs = NEW * CACHED + NEW * (NEW + 1) // 2            # visible (query, key) pairs per head
     flops = pairs * D * 2 * 2 * HQ * S                     # QK^T and PV, 2 flops per MAC
@@ -548,6 +563,15 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the auxiliary measurements (KV store, fused q/k kernel, sampler, model step): "
                          "keeps a profiler trace of the run small")
+    ap.add_argument("--min-launches", type=int, default=MIN_LAUNCHES,
+                    help="launches per timed repeat are max(steps, this); profiler runs with counters lower it")
+    ap.add_argument("--sections", default="all",
+                    help="comma-separated parts to run: headline (the FP16 / FP8 launches), probe (the same "
+                         "launches with loads only), others (configs 1, 3, 4 and the wider GQA groups), prefill, "
+                         "extras, cpu; 'all' = every one.  For profiler runs, which want one kind of launch "
+                         "per kernel name: the load probe is the decode kernel itself with a flag set, and the "
+                         "other configurations launch the headline's kernels on other shapes.  Without "
+                         "`headline` the run prints a reduced line for the parts it ran")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device-to-device copies (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
@@ -558,6 +582,32 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    sections = set(args.sections.split(","))
+    if "all" in sections:
+        sections = {"headline", "probe", "others", "prefill", "extras", "cpu"}
+    if args.no_extras:
+        sections.discard("extras")
+    if args.no_cpu_baseline:
+        sections.discard("cpu")
+    unknown = sections - {"headline", "probe", "others", "prefill", "extras", "cpu"}
+    if unknown:
+        print("bench.py: unknown section(s) %s" % sorted(unknown), file=sys.stderr)
+        sys.exit(2)
+    if not sections & {"headline", "probe", "cpu"}:
+        # profiler runs of the other parts alone: their kernels share names with the headline's
+        import torch
+        import ai_infra_train_infer_amd as pa
+        dev = torch.device("cuda:0")
+        torch.cuda.set_device(dev)
+        launches = max(args.steps, args.min_launches)
+        part = {"sections": sorted(sections)}
+        if "others" in sections:
+            part["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+        if "prefill" in sections:
+            part["prefill_mfma"] = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup))
+        print(json.dumps(part))
+        return
+    probe_only = "headline" not in sections and "cpu" not in sections
     import torch
     import ai_infra_train_infer_amd as pa
     lib = pa._native.load()
@@ -576,7 +626,7 @@ def main():
 
     B, CTX, HQ, HKV, D, BS = args.batch, args.ctx, 16, 8, 128, 16
     scale = 1.0 / math.sqrt(D)
-    launches = max(args.steps, MIN_LAUNCHES)
+    launches = max(args.steps, args.min_launches)
     stream = torch.cuda.current_stream(dev).cuda_stream
     work, fns, shape = {}, {}, {}
     for kind in ("fp16", "fp8"):
@@ -592,7 +642,8 @@ def main():
             pa.paged_decode(w["q"], w["k_cache"], w["v_cache"], w["block_tables"],
                             w["context_lens"], scale, w["k_scale"], w["v_scale"], out=w["out"])
 
-        fns[kind] = step
+        if not probe_only:
+            fns[kind] = step
         # the same launch with the arithmetic taken out: what the memory system needs for this
         # access pattern alone
         pbytes = lib.pa_workspace_bytes(B, HQ, D, parts)
@@ -608,8 +659,9 @@ def main():
                 w["probe_ws"].numel(), 0, hpw, 0, stream)
             assert rc == 0, lib.pa_last_error()
 
-        fns[kind + "_probe"] = probe
-        if parts > 1:
+        if "probe" in sections:
+            fns[kind + "_probe"] = probe
+        if parts > 1 and not probe_only:
             # dominant kernel alone: the attention pass without the merge (a single-pass launch IS
             # that one kernel, so its operator timing is used as it stands)
             nbytes = lib.pa_workspace_bytes(B, HQ, D, parts)
@@ -627,6 +679,10 @@ def main():
 
             fns[kind + "_kernel"] = kernel_only
 
+    if probe_only:
+        t = time_alternating(torch, fns, launches)
+        print(json.dumps({"sections": ["probe"], "loads_only_us": {k: spread(v) for k, v in t.items()}}))
+        return
     # the W untimed + K timed steps the command line asked for, on the host clock: what an outside
     # stopwatch around this process sees of one pass
     _, wall_ms = time_steps(torch, fns["fp16"], args.steps, args.warmup)
@@ -637,10 +693,10 @@ def main():
         k_us = t.get(kind + "_kernel", us)
         assert med(k_us) <= med(us) * 1.02, "the attention pass alone cannot take longer than the call that contains it"
         nbytes_alg = algorithmic_bytes(B, CTX, HQ, HKV, D, BS, kind == "fp8")
-        results[kind] = dict(us=us, kernel_us=k_us, bytes=nbytes_alg, probe_us=t[kind + "_probe"],
+        results[kind] = dict(us=us, kernel_us=k_us, bytes=nbytes_alg, probe_us=t.get(kind + "_probe"),
                              gbps=nbytes_alg / med(us) / 1e3, kernel_gbps=nbytes_alg / min(med(k_us), med(us)) / 1e3,
                              partition_size=shape[kind][0], partitions=shape[kind][1], kv_heads_per_wave=shape[kind][2])
-    if not args.no_cpu_baseline:
+    if "cpu" in sections:
         w = work["fp16"]
         n = min(args.cpu_sample_seqs, B)
         sec, cpu_out = cpu_baseline(torch, w, scale, n, BS)
@@ -658,7 +714,7 @@ def main():
     del work, fns, w
     torch.cuda.empty_cache()
 
-    prefill = prefill_cfg5a(pa, torch, dev, max(50, args.steps), max(20, args.warmup))   # the first launches run below the steady rate
+    prefill = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup)) if "prefill" in sections else None
     f16, f8 = results["fp16"], results["fp8"]
     speedup = med(f16["us"]) / med(f8["us"])
     line = {
@@ -710,18 +766,21 @@ def main():
             "fp8_kernel": {"achieved": round(f8["kernel_gbps"], 1), "frac": round(f8["kernel_gbps"] / HBM_PEAK_GBPS, 4),
                            "algorithmic_bytes": f8["bytes"],
                            "traffic": measured_traffic("traffic_bytes_fp8") if (B, CTX) == (64, 4096) else None},
-            "loads_only": {
-                "what": "pa_decode_load_probe: the same launches with every load issued and consumed but no "
-                        "attention arithmetic, i.e. the rate the memory system gives this access pattern",
-                "fp16_us": spread(f16["probe_us"]), "fp16_gbps": round(f16["bytes"] / med(f16["probe_us"]) / 1e3, 1),
-                "fp8_us": spread(f8["probe_us"]), "fp8_gbps": round(f8["bytes"] / med(f8["probe_us"]) / 1e3, 1),
-                "fp16_kernel_vs_loads_only": round(med(f16["probe_us"]) / min(med(f16["kernel_us"]), med(f16["us"])), 3),
-                "fp8_kernel_vs_loads_only": round(med(f8["probe_us"]) / min(med(f8["kernel_us"]), med(f8["us"])), 3)},
         },
     }
-    line["other_configs"] = other_decode_configs(pa, torch, dev, launches)
-    line["prefill_mfma"] = prefill
-    if not args.no_extras:
+    if "probe" in sections:
+        line["roofline"]["loads_only"] = {
+            "what": "pa_decode_load_probe: the same launches with every load issued and consumed but no "
+                    "attention arithmetic, i.e. the rate the memory system gives this access pattern",
+            "fp16_us": spread(f16["probe_us"]), "fp16_gbps": round(f16["bytes"] / med(f16["probe_us"]) / 1e3, 1),
+            "fp8_us": spread(f8["probe_us"]), "fp8_gbps": round(f8["bytes"] / med(f8["probe_us"]) / 1e3, 1),
+            "fp16_kernel_vs_loads_only": round(med(f16["probe_us"]) / min(med(f16["kernel_us"]), med(f16["us"])), 3),
+            "fp8_kernel_vs_loads_only": round(med(f8["probe_us"]) / min(med(f8["kernel_us"]), med(f8["us"])), 3)}
+    if "others" in sections:
+        line["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+    if prefill is not None:
+        line["prefill_mfma"] = prefill
+    if "extras" in sections:
         line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
         line["kv_gather"] = kv_gather_times(pa, torch, dev, args.steps, args.warmup)
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
