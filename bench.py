@@ -295,9 +295,12 @@ def other_decode_configs(pa, torch, dev, launches):
     return out
 
 
-def prefill_cfg5a(pa, torch, dev, steps, warmup):
+def prefill_cfg5a(pa, torch, dev, steps, warmup, constant_data=False):
     """Fifth benchmark configuration, first half: 8 sequences x (2048 cached + 512 new tokens), bf16 Q, FP16
-    KV, causal within the chunk; judged against the dense fp16 MFMA peak."""
+    KV, causal within the chunk; judged against the dense fp16 MFMA peak.  constant_data: the same
+    launch with Q, K and V all ones - the same instruction stream on operands that do not toggle,
+    which shows how much of the time the GPU's power management takes (clocks drop under the
+    matrix pipe on random data)."""
     S, CACHED, NEW, HQ, HKV, D, BS = 8, 2048, 512, 16, 8, 128, 16
     g = torch.Generator(device=dev).manual_seed(1005)
     bps = (CACHED + NEW) // BS
@@ -309,6 +312,10 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup):
     cu_q = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * NEW
     cu_k = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * (CACHED + NEW)
     out = torch.empty_like(q)
+    if constant_data:
+        q.fill_(1.0)
+        kc.fill_(1.0)
+        vc.fill_(1.0)
 
     def step():
         pa.paged_prefill(q, kc, vc, cu_q, cu_k, NEW, D ** -0.5, block_tables=tables, out=out)
@@ -781,6 +788,11 @@ def main():
     if prefill is not None:
         line["prefill_mfma"] = prefill
     if "extras" in sections:
+        const = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup), constant_data=True)
+        line["prefill_mfma_constant_operands"] = {
+            "what": "the prefill launch above with Q, K and V all ones: the same instructions on operands that do "
+                    "not toggle; the difference to `prefill_mfma` is clock throttling under the matrix pipe",
+            "us": const["us"], "tflops": const["tflops"], "frac_mfma_peak": const["frac_mfma_peak"]}
         line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
         line["kv_gather"] = kv_gather_times(pa, torch, dev, args.steps, args.warmup)
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
