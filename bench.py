@@ -330,6 +330,39 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup, constant_data=False):
             "frac_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
 
 
+def mfma_ceiling(pa, torch, dev):
+    """What the matrix pipe sustains on this GPU: pa_mfma_rate_probe (independent
+    v_mfma_f32_32x32x16_f16 on every SIMD, operands from registers, launches of ~10 ms) on constant
+    operands and on N(0,1) operands, alternated, median of 5.  The clocks drop under the matrix
+    pipe, further when the operands toggle, so the nominal dense-fp16 peak is not a sustained rate."""
+    lib = pa._native.load()
+    g = torch.Generator(device=dev).manual_seed(14)
+    ops = {"constant_operands": torch.ones(65536, dtype=torch.float16, device=dev),
+           "normal_operands": torch.randn(65536, generator=g, device=dev, dtype=torch.float32).half()}
+    sink = torch.empty(1024, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    steps = 20000
+    res = {k: [] for k in ops}
+    flops = 0
+    for rep_ in range(6):
+        for name, t in ops.items():
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            flops = lib.pa_mfma_rate_probe(t.data_ptr(), steps, sink.data_ptr(), stream)
+            stop.record()
+            torch.cuda.synchronize()
+            assert flops > 0, lib.pa_last_error()
+            if rep_:
+                res[name].append(start.elapsed_time(stop))
+    out = {"what": "pa_mfma_rate_probe: nothing but independent v_mfma_f32_32x32x16_f16 on every SIMD, "
+                   "8 waves per CU, launches of 10-15 ms", "nominal_peak_tflops": 2500.0}
+    for name, v in res.items():
+        ms = sorted(v)[len(v) // 2]
+        out[name] = {"ms": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
+                     "frac_of_nominal": round(flops / ms / 1e9 / 2500.0, 4)}
+    return out
+
+
 def kv_store_times(pa, torch, dev, steps, warmup):
     """Paged KV-cache write of one decode step (64 new tokens) and of one prefill chunk (4096
     tokens), FP16 copy and FP8 quantising store.  Latency-bound: reported in microseconds only."""
@@ -789,6 +822,10 @@ def main():
         line["prefill_mfma"] = prefill
     if "extras" in sections:
         const = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup), constant_data=True)
+        line["mfma_sustained"] = mfma_ceiling(pa, torch, dev)
+        if prefill is not None:
+            line["prefill_mfma"]["frac_of_sustained_mfma_rate_on_normal_operands"] = round(
+                prefill["tflops"] / line["mfma_sustained"]["normal_operands"]["tflops"], 4)
         line["prefill_mfma_constant_operands"] = {
             "what": "the prefill launch above with Q, K and V all ones: the same instructions on operands that do "
                     "not toggle; the difference to `prefill_mfma` is clock throttling under the matrix pipe",

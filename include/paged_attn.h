@@ -210,6 +210,17 @@ int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride, con
                          void* stream);
 
 /*
+ * Measuring aid: the rate the matrix pipe sustains.  Runs nothing but independent
+ * v_mfma_f32_32x32x16_f16 on every SIMD (one workgroup of 8 waves per compute unit, `steps` x 16
+ * products per wave) on operands taken from `operands_f16` (65536 fp16 values: constants, or the
+ * kind of data the attention kernels see - the clocks of the part depend on how the operands
+ * toggle).  `sink` receives one float per compute unit (at least 1024 floats).  Returns the number
+ * of floating-point operations of the launch (time it with events on `stream`), or a negative
+ * error code.  No counterpart in the reference.
+ */
+int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t steps, float* sink, void* stream);
+
+/*
  * Merge reduction over partitions.
  * Replaces: PartitionedPagedAttention._merge_partitions (src/inference/attention.py:591-626).
  * out = sum_p w_p * out_p / sum_p w_p with w_p = sum_p * exp(max_p - max_all), over the

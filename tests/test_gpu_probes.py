@@ -1,0 +1,48 @@
+"""The two measuring aids of the library run and report what they say they do: the decode launch
+with its arithmetic taken out (pa_decode_load_probe) and the matrix-pipe rate probe
+(pa_mfma_rate_probe).  Their timings belong to bench.py; here only the contracts are checked."""
+import pytest
+import torch
+
+import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def test_mfma_rate_probe_counts_its_work_and_rejects_bad_arguments(pa, lib, gpu):
+    ops = torch.ones(65536, dtype=torch.float16, device=gpu)
+    sink = torch.full((1024,), float("nan"), dtype=torch.float32, device=gpu)
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    flops = lib.pa_mfma_rate_probe(ops.data_ptr(), 4, sink.data_ptr(), stream)
+    torch.cuda.synchronize()
+    assert flops == cus * 8 * 4 * 16 * 32768
+    got = sink[:cus].cpu()
+    # all-ones operands: every product adds 16 to each element of its accumulator; 4 steps x 16 products over 4
+    # chains = 16 products per chain = 256 per element; the sink sums two elements of each of the 4 chains
+    assert torch.all(got == 4 * 2 * 256.0), got[:4]
+    assert torch.isnan(sink[cus:]).all()
+    assert lib.pa_mfma_rate_probe(None, 4, sink.data_ptr(), stream) == -1
+    assert lib.pa_mfma_rate_probe(ops.data_ptr(), 0, sink.data_ptr(), stream) == -1
+    assert b"steps" in lib.pa_last_error()
+
+
+def test_decode_load_probe_runs_the_decode_launch_shape(pa, lib, gpu):
+    lens = cases.uniform_lens(5, 8, 128, 512)
+    c = cases.make_case(1001, lens, 512, cache="fp8")
+    d = cases.to_device(c, gpu)
+    ws = torch.zeros(lib.pa_workspace_bytes(8, 16, 128, 4), dtype=torch.uint8, device=gpu)
+    rc = lib.pa_decode_load_probe(
+        d["q"].data_ptr(), 0, 16 * 128, d["k_cache"].data_ptr(), d["v_cache"].data_ptr(), d["k_scale"].data_ptr(),
+        d["v_scale"].data_ptr(), pa._native.DTYPE_FP8_E4M3, d["block_tables"].data_ptr(), d["block_tables"].stride(0),
+        d["block_tables"].shape[1], d["context_lens"].data_ptr(), 8, 16, 8, 128, 16, c["num_blocks"], 128, 4,
+        ws.data_ptr(), ws.numel(), 0, 0, 0, torch.cuda.current_stream(gpu).cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0, lib.pa_last_error()
+    # too small a workspace is refused like in the real launch
+    rc = lib.pa_decode_load_probe(
+        d["q"].data_ptr(), 0, 16 * 128, d["k_cache"].data_ptr(), d["v_cache"].data_ptr(), d["k_scale"].data_ptr(),
+        d["v_scale"].data_ptr(), pa._native.DTYPE_FP8_E4M3, d["block_tables"].data_ptr(), d["block_tables"].stride(0),
+        d["block_tables"].shape[1], d["context_lens"].data_ptr(), 8, 16, 8, 128, 16, c["num_blocks"], 128, 4,
+        ws.data_ptr(), 256, 0, 0, 0, torch.cuda.current_stream(gpu).cuda_stream)
+    assert rc == -4
