@@ -330,6 +330,37 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup, constant_data=False):
             "frac_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
 
 
+def hbm_stream_read(pa, torch, dev, launches):
+    """The plain read rate of the GPU: pa_hbm_read_probe over a 1 GiB buffer (every workgroup streams
+    its own contiguous share once, 16-byte loads), for four workgroup counts, alternated, medians.
+    1 GiB exceeds the 256 MB of last-level cache, so every launch reads HBM."""
+    lib = pa._native.load()
+    nbytes = 1 << 30
+    buf = torch.ones(nbytes // 4, dtype=torch.float32, device=dev)
+    sink = torch.empty(1 << 15, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    cus = pa.attention._compute_units(dev)
+    fns = {}
+    for mult in (2, 8, 32, 128):
+        groups = cus * mult
+
+        def fn(groups=groups):
+            got = lib.pa_hbm_read_probe(buf.data_ptr(), nbytes, groups, sink.data_ptr(), stream)
+            assert got == nbytes, lib.pa_last_error()
+
+        fns["workgroups_%d" % groups] = fn
+    t = time_alternating(torch, fns, max(20, launches // 5), warmup=3)
+    out = {"what": "pa_hbm_read_probe: 1 GiB streamed once per launch, contiguous share per workgroup, 16-byte loads",
+           "bytes": nbytes}
+    for name, v in t.items():
+        out[name] = {"us": spread(v), "gbps": round(nbytes / med(v) / 1e3, 1),
+                     "frac_of_8TBps": round(nbytes / med(v) / 1e3 / HBM_PEAK_GBPS, 4)}
+    out["best_gbps"] = max(v["gbps"] for k, v in out.items() if k.startswith("workgroups_"))
+    del buf
+    torch.cuda.empty_cache()
+    return out
+
+
 def mfma_ceiling(pa, torch, dev):
     """What the matrix pipe sustains on this GPU: pa_mfma_rate_probe (independent
     v_mfma_f32_32x32x16_f16 on every SIMD, operands from registers, launches of ~10 ms) on constant
@@ -721,7 +752,10 @@ def main():
 
     if probe_only:
         t = time_alternating(torch, fns, launches)
-        print(json.dumps({"sections": ["probe"], "loads_only_us": {k: spread(v) for k, v in t.items()}}))
+        del work, fns
+        torch.cuda.empty_cache()
+        print(json.dumps({"sections": ["probe"], "loads_only_us": {k: spread(v) for k, v in t.items()},
+                          "hbm_stream_read": hbm_stream_read(pa, torch, dev, launches)}))
         return
     # the W untimed + K timed steps the command line asked for, on the host clock: what an outside
     # stopwatch around this process sees of one pass
@@ -816,6 +850,10 @@ def main():
             "fp8_us": spread(f8["probe_us"]), "fp8_gbps": round(f8["bytes"] / med(f8["probe_us"]) / 1e3, 1),
             "fp16_kernel_vs_loads_only": round(med(f16["probe_us"]) / min(med(f16["kernel_us"]), med(f16["us"])), 3),
             "fp8_kernel_vs_loads_only": round(med(f8["probe_us"]) / min(med(f8["kernel_us"]), med(f8["us"])), 3)}
+        stream_read = hbm_stream_read(pa, torch, dev, launches)
+        line["roofline"]["hbm_stream_read"] = stream_read
+        line["roofline"]["frac_of_plain_stream_read"] = round(f16["kernel_gbps"] / stream_read["best_gbps"], 4)
+        line["roofline"]["fp8_kernel"]["frac_of_plain_stream_read"] = round(f8["kernel_gbps"] / stream_read["best_gbps"], 4)
     if "others" in sections:
         line["other_configs"] = other_decode_configs(pa, torch, dev, launches)
     if prefill is not None:

@@ -221,6 +221,14 @@ int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride, con
 int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t steps, float* sink, void* stream);
 
 /*
+ * Measuring aid: the plain read rate of the GPU.  `groups` workgroups of 256 threads each stream
+ * their own contiguous share of `bytes` bytes at `src` once (16-byte loads, four per lane in flight)
+ * and leave the XOR of their words, folded to 32 bits, in sink[group].  Returns the number of bytes
+ * read (bytes rounded down to 16 x groups), or a negative error code.  No counterpart in the reference.
+ */
+int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, uint32_t* sink, void* stream);
+
+/*
  * Merge reduction over partitions.
  * Replaces: PartitionedPagedAttention._merge_partitions (src/inference/attention.py:591-626).
  * out = sum_p w_p * out_p / sum_p w_p with w_p = sum_p * exp(max_p - max_all), over the
