@@ -23,7 +23,7 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
             f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
-            "-I", INCLUDE, "-I", CSRC] + DEVICE_FLAGS
+            "-I", INCLUDE, "-I", CSRC, "-Rpass-analysis=kernel-resource-usage"] + DEVICE_FLAGS
 
 
 def _hipcc():
@@ -53,9 +53,30 @@ def _compile(hipcc, src):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr[-8000:]))
+    # No kernel of the library may use scratch memory (register spills or arrays the compiler could not
+    # keep in registers): such a kernel is several times slower than intended and nothing else says so.
+    name, spilled = "?", []
+    for ln in r.stderr.splitlines():
+        if "Function Name:" in ln:
+            name = ln.split("Function Name:")[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in ln:
+            size = int(ln.split("ScratchSize [bytes/lane]:")[1].split()[0])
+            if size:
+                spilled.append("%s: %d bytes of scratch per lane" % (name, size))
+    if spilled:
+        raise RuntimeError("kernels of %s use scratch memory:\n%s" % (src, "\n".join(spilled)))
     # the host pass does not know the device-only target feature; that warning is expected
     noise = ("packed-fp32-ops", "is not a recognized feature")
-    msgs = [ln for ln in r.stderr.splitlines() if ln.strip() and not any(n in ln for n in noise)]
+    msgs, skip = [], 0
+    for ln in r.stderr.splitlines():
+        if "kernel-resource-usage" in ln:
+            skip = 2          # the remark's source line and caret follow it
+        elif skip and (ln.lstrip()[:1].isdigit() or ln.lstrip().startswith("|")):
+            skip -= 1
+        else:
+            skip = 0
+            if ln.strip() and not ln.startswith("In file included from") and not any(n in ln for n in noise):
+                msgs.append(ln)
     return obj, "\n".join(msgs)
 
 
