@@ -470,6 +470,7 @@ _CU_BYTES_PER_NS = {2: 31.0, 1: 22.0}      # by cache element size: fp8 rows cos
 _ROUND_NS = 2000.0
 _MERGE_NS = (5000.0, 250.0)        # fixed, per partition (the pass itself and the partials it re-reads)
 _DEFAULT_COMPUTE_UNITS = 256
+MATRIX_PATH_FROM_RATIO = 3         # GQA ratio from which pa_decode multiplies on the matrix cores (up to 16 query heads per workgroup)
 _CU_COUNT = {}
 
 
@@ -505,10 +506,15 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
     if max_context <= _MIN_AUTO_PARTITION or batch <= 0:
         return 0, 1
     g = num_q_heads // num_kv_heads
-    gc = 2 if g % 2 == 0 else 1
-    can_pair = g == gc and num_kv_heads % 2 == 0
+    if g >= MATRIX_PATH_FROM_RATIO:
+        # the matrix kernel: one workgroup per KV head and slice of 16 query heads
+        units = batch * num_kv_heads * -(-g // 16)
+        can_pair = num_kv_heads % 2 == 0
+    else:
+        gc = 2 if g % 2 == 0 else 1
+        can_pair = g == gc and num_kv_heads % 2 == 0
+        units = batch * (num_q_heads // gc)              # workgroups of one partition, unpaired
     narrow = head_dim * kv_elem_bytes <= 128
-    units = batch * (num_q_heads // gc)                  # workgroups of one partition, unpaired
     token_bytes = 2.0 * head_dim * kv_elem_bytes         # K and V of one head
     cu_rate = _CU_BYTES_PER_NS.get(kv_elem_bytes, 31.0)
     hbm_ns = batch * num_kv_heads * max_context * token_bytes / _HBM_BYTES_PER_NS

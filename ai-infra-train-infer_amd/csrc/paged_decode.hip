@@ -136,6 +136,9 @@ static int scratch_for_current_device(void** out) {
 
 enum { kDecodeFull = 0, kDecodePartials = 1, kDecodeProbe = 2 };
 
+constexpr int kMatrixPath = 16;            // q_heads_per_wave value that names the MFMA kernel
+constexpr int kMatrixPathFromRatio = 3;     // GQA ratio from which the automatic choice takes it
+
 // Shared argument checking + launch of the attention pass; `merge` adds the reduction.
 static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_token_stride,
                        const void* k_cache, const void* v_cache, const float* k_scale,
@@ -194,8 +197,9 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   if (kv_heads_per_wave != 0 && kv_heads_per_wave != 1 && kv_heads_per_wave != 2 &&
       kv_heads_per_wave != 4 && kv_heads_per_wave != 8)
     PA_FAIL(PA_ERR_BAD_ARG, "kv_heads_per_wave must be 0 (automatic), 1, 2, 4 or 8");
-  if (q_heads_per_wave != 0 && q_heads_per_wave != 1 && q_heads_per_wave != 2 && q_heads_per_wave != 4)
-    PA_FAIL(PA_ERR_BAD_ARG, "q_heads_per_wave must be 0 (automatic), 1, 2 or 4");
+  if (q_heads_per_wave != 0 && q_heads_per_wave != 1 && q_heads_per_wave != 2 && q_heads_per_wave != 4 &&
+      q_heads_per_wave != kMatrixPath)
+    PA_FAIL(PA_ERR_BAD_ARG, "q_heads_per_wave must be 0 (automatic), 1, 2, 4 or 16 (the matrix path)");
   const bool direct = merge && max_partitions == 1;
   if (!direct) {
     if (max_partitions > 1 && (partition_size <= 0 || partition_size % 16 != 0))
@@ -214,36 +218,67 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   const int g = (int)(num_q_heads / num_kv_heads);
   DecodeShape s;
   s.head_dim = (int)head_dim;
-  if (q_heads_per_wave != 0) {
-    if (g % q_heads_per_wave != 0) PA_FAIL(PA_ERR_UNSUPPORTED, "q_heads_per_wave must divide num_q_heads / num_kv_heads");
-    s.gc = q_heads_per_wave;
+  int slices;                                 // workgroups per KV head
+  // The matrix path (paged_decode_mfma_kernel.hpp) takes up to 16 query heads of a KV head as one
+  // MFMA operand: the choice from a GQA ratio of 3 on, where the vector kernel's arithmetic per
+  // loaded byte starts to cost more than the loads (batch 64 x 4096 tokens, fp16 / fp8 cache: ratio 4
+  // 187 / 103 us against 195 / 142 us, ratio 8 187 / 103 against 239 / 257, ratio 2 182 / 100.5 against 179 / 100).
+  bool matrix = q_heads_per_wave == kMatrixPath;
+  if (q_heads_per_wave == 0 && g >= kMatrixPathFromRatio && mode != kDecodeProbe && kv_heads_per_wave <= 2 &&
+      (waves == 0 || waves >= 2) && !(kv_heads_per_wave == 2 && (waves == 8 || num_kv_heads % 2 != 0)))
+    matrix = true;
+  if (matrix) {
+    if (mode == kDecodeProbe) PA_FAIL(PA_ERR_UNSUPPORTED, "the load probe follows the vector kernel: q_heads_per_wave 1, 2 or 4");
+    if (kv_heads_per_wave > 2 || (kv_heads_per_wave == 2 && num_kv_heads % 2 != 0))
+      PA_FAIL(PA_ERR_UNSUPPORTED, "the matrix path takes one KV head per wave, or two of an even number");
+    if (waves == 1 || (kv_heads_per_wave == 2 && waves == 8))
+      PA_FAIL(PA_ERR_UNSUPPORTED, "the matrix path takes 2, 4 or 8 waves per workgroup with one KV head per wave, 2 or 4 with two");
+    s.gc = kMatrixPath;
+    s.qs = 1;
+    slices = (g + kMatrixPath - 1) / kMatrixPath;
+    // One KV head per wave.  4-wave workgroups (two share a CU) are the best or within 3 % of the best
+    // shape from batch 8 x 320 to batch 256 x 1k tokens; launches with fewer workgroups than CUs put
+    // 8 waves on the CUs they do reach.  Two heads per wave gain nothing here: the wave's longer
+    // chain of products per tile costs what the wider pieces save.
+    s.hpw = kv_heads_per_wave == 2 ? 2 : 1;
+    if (waves != 0) {
+      s.waves = waves;
+    } else {
+      const int64_t wgs = (num_kv_heads / s.hpw) * slices * max_partitions * batch;
+      s.waves = (s.hpw == 1 && wgs < compute_units()) ? 8 : 4;
+    }
   } else {
-    s.gc = (g % 4 == 0) ? 4 : (g % 2 == 0) ? 2 : 1;
-  }
-  const int rest = g / s.gc;
-  const int split_waves = s.gc == 4 ? 4 : 8;
-  s.qs = 1;
-  if (s.gc >= 2 && rest % 2 == 0 && (waves == 0 || waves == split_waves)) s.qs = (rest % 4 == 0) ? 4 : 2;
-  const int slices = rest / s.qs;           // workgroups per KV head
-  s.waves = s.qs > 1 ? split_waves : (waves == 0 ? 4 : waves);
-  // Several adjacent KV heads per wave need each KV head's query group whole in the wave.
-  const bool can_share = g == s.gc && s.gc <= 2;
-  s.hpw = 1;
-  if (kv_heads_per_wave > 1) {
-    if (!can_share || num_kv_heads % kv_heads_per_wave != 0 ||
-        (kv_heads_per_wave > 2 && (s.gc != 2 || (s.waves != 4 && s.waves != 8))))
-      PA_FAIL(PA_ERR_UNSUPPORTED, "kv_heads_per_wave does not fit this head layout");
-    s.hpw = kv_heads_per_wave;
-  } else if (kv_heads_per_wave == 0 && can_share && num_kv_heads % 2 == 0) {
-    // Two heads per wave when halving the workgroups does not add a round of them over the CUs: a
-    // CU streams at a fixed rate however many workgroups it hosts, the launch takes as long as
-    // its busiest CU, and fewer, longer-lived workgroups stream better (185 -> 178 us at batch 64 /
-    // ctx 4096, fp16; rows of 128 bytes or less gain another 10% from being read as 256-byte
-    // pieces).  With a workgroup or less per CU pairing would only idle CUs.
-    const int64_t cus = compute_units();
-    const int64_t wgs = num_kv_heads * max_partitions * batch;      // unpaired
-    const int64_t rounds = (wgs + cus - 1) / cus, paired_rounds = (wgs + 2 * cus - 1) / (2 * cus);
-    if (wgs >= 8 * cus || 2 * paired_rounds <= rounds) s.hpw = 2;
+    if (q_heads_per_wave != 0) {
+      if (g % q_heads_per_wave != 0) PA_FAIL(PA_ERR_UNSUPPORTED, "q_heads_per_wave must divide num_q_heads / num_kv_heads");
+      s.gc = q_heads_per_wave;
+    } else {
+      s.gc = (g % 4 == 0) ? 4 : (g % 2 == 0) ? 2 : 1;
+    }
+    const int rest = g / s.gc;
+    const int split_waves = s.gc == 4 ? 4 : 8;
+    s.qs = 1;
+    if (s.gc >= 2 && rest % 2 == 0 && (waves == 0 || waves == split_waves)) s.qs = (rest % 4 == 0) ? 4 : 2;
+    slices = rest / s.qs;
+    s.waves = s.qs > 1 ? split_waves : (waves == 0 ? 4 : waves);
+    // Several adjacent KV heads per wave need each KV head's query group whole in the wave.
+    const bool can_share = g == s.gc && s.gc <= 2;
+    s.hpw = 1;
+    if (kv_heads_per_wave > 1) {
+      if (!can_share || num_kv_heads % kv_heads_per_wave != 0 ||
+          (kv_heads_per_wave > 2 && (s.gc != 2 || (s.waves != 4 && s.waves != 8))))
+        PA_FAIL(PA_ERR_UNSUPPORTED, "kv_heads_per_wave does not fit this head layout");
+      s.hpw = kv_heads_per_wave;
+    } else if (kv_heads_per_wave == 0 && can_share && num_kv_heads % 2 == 0) {
+      // Two heads per wave when halving the workgroups does not add a round of them over the CUs: a
+      // CU streams at a fixed rate however many workgroups it hosts, the launch takes as long as
+      // its busiest CU, and fewer, longer-lived workgroups stream better (185 -> 178 us at batch 64 /
+      // ctx 4096, fp16; rows of 128 bytes or less gain another 10% from being read as 256-byte
+      // pieces).  With a workgroup or less per CU pairing would only idle CUs.
+      const int64_t cus = compute_units();
+      const int64_t wgs = num_kv_heads * max_partitions * batch;      // unpaired
+      const int64_t rounds = (wgs + cus - 1) / cus, paired_rounds = (wgs + 2 * cus - 1) / (2 * cus);
+      if (wgs >= 8 * cus || 2 * paired_rounds <= rounds) s.hpw = 2;
+    }
   }
 #undef PA_FAIL
 

@@ -1,6 +1,6 @@
 // Instantiations of the paged decode kernel for fp8 caches (one translation unit per cache
 // element type, so that the three compile side by side).
-#include "paged_decode_kernel.hpp"
+#include "paged_decode_mfma_kernel.hpp"
 
 namespace pa {
 

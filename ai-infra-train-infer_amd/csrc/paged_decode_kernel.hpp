@@ -71,7 +71,7 @@ struct DecodeParams {
 // How a launch is cut: all fields are template parameters of the kernel it selects.
 struct DecodeShape {
   int head_dim;   // 64 or 128
-  int gc;         // query heads per wave and KV head: 1, 2 or 4
+  int gc;         // query heads per wave and KV head: 1, 2 or 4; 16 = the matrix kernel (up to 16 as one MFMA operand)
   int hpw;        // KV heads per wave: 1, 2, 4 or 8
   int qs;         // wave groups over the same tokens, each with its own gc query heads: 1, 2 or 4
   int waves;      // waves per workgroup (all groups together): 1, 2, 4 or 8
@@ -611,7 +611,11 @@ static int launch_decode_dim(const DecodeParams& p, dim3 grid, const DecodeShape
 }
 
 template <int KV>
+static int launch_decode_mfma(const DecodeParams& p, dim3 grid, const DecodeShape& s, hipStream_t st);
+
+template <int KV>
 static int launch_decode_kv(const DecodeParams& p, dim3 grid, const DecodeShape& s, hipStream_t st) {
+  if (s.gc == 16) return launch_decode_mfma<KV>(p, grid, s, st);
   if (s.head_dim == 128) return launch_decode_dim<KV, 128>(p, grid, s, st);
   if (s.head_dim == 64) return launch_decode_dim<KV, 64>(p, grid, s, st);
   return fail(PA_ERR_UNSUPPORTED, "pa_decode: head_dim must be 64 or 128");

@@ -135,7 +135,11 @@ int64_t pa_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t head_dim,
  *   q_heads_per_wave     0 = the launch's own choice, or 1, 2, 4 (a divisor of the GQA ratio):
  *                        query heads of a KV head held in one wave's registers; the rest of the
  *                        ratio goes to groups of waves inside the workgroup (factors 2 and 4)
- *                        and, beyond that, to separate workgroups.
+ *                        and, beyond that, to separate workgroups.  16 = the matrix kernel: up
+ *                        to 16 query heads of a KV head (any ratio; wider groups in slices of 16)
+ *                        as one MFMA operand, the launch's own choice from a ratio of 3 on; it
+ *                        takes 2, 4 or 8 waves and kv_heads_per_wave 1, or 2 (of an even number
+ *                        of KV heads, with 2 or 4 waves).
  *                        The result does not depend on any of the three.
  */
 int pa_decode(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,

@@ -252,7 +252,9 @@ def test_c_abi_argument_errors(lib, gpu):
     assert call(parts=4, psize=500, ws=p, wsb=1 << 30) == -2      # not a multiple of 16
     assert call(parts=4, psize=512) == -4         # workspace missing
     assert call(waves=3) == -1 and call(hpw=3) == -1 and call(qpw=3) == -1
-    assert call(hq=32, hpw=2) == -2               # several KV heads per wave need a GQA ratio <= 2
+    assert call(hq=32, hpw=2, qpw=4) == -2        # the vector kernel: several KV heads per wave need a GQA ratio <= 2
+    assert call(hq=32, hpw=4) == -2 and call(hq=32, qpw=16, waves=1) == -2     # the matrix kernel: 1 or 2 heads, 2+ waves
+    assert call(hq=32, qpw=16, hpw=2, waves=8) == -2
     assert call(hq=32, qpw=8) == -1 and call(hq=24, hkv=8, qpw=2) == -2
     assert call(hpw=4, waves=2) == -2
 
@@ -363,3 +365,68 @@ def test_workspace_is_per_device_grows_outside_captures_and_outlives_graphs(pa, 
                         dl["scale"], partition_size=64)
         torch.cuda.synchronize()
     del junk
+
+
+# ---- the matrix kernel (q_heads_per_wave = 16; the launch's own choice from a GQA ratio of 3) -------
+
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (64, 8, 128), (16, 8, 128), (8, 8, 128), (12, 4, 128),
+                                       (40, 8, 64), (48, 2, 64), (40, 2, 128), (34, 2, 128)])
+@pytest.mark.parametrize("cache", ["fp16", "fp8", "bf16"])
+def test_matrix_kernel_head_shapes(pa, gpu, hq, hkv, d, cache):
+    """Ratios 1 ... 24 (more than 16 query heads per KV head run as slices of 16, the last one ragged),
+    one and two KV heads per wave, every workgroup width, single pass and partitions."""
+    lens = [3, 200, 1025, 77, 32, 33, 64, 1]
+    c = cases.make_case(hq + d, lens, 128, num_heads=hq, num_kv_heads=hkv, head_dim=d, cache=cache,
+                        q_dtype=torch.bfloat16 if cache == "bf16" else torch.float16)
+    want = oracle_decode(c)
+    for kw in (dict(), dict(partition_size=256), dict(waves=4), dict(waves=2, partition_size=48),
+               dict(kv_heads_per_wave=2), dict(kv_heads_per_wave=2, waves=2, partition_size=80),
+               dict(kv_heads_per_wave=1, waves=8, partition_size=32)):
+        check(gpu_decode(pa, c, gpu, q_heads_per_wave=16, **kw), want, cache)
+
+
+@pytest.mark.parametrize("bs", [8, 32, 128])
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_matrix_kernel_block_sizes_and_empty_rows(pa, gpu, bs, cache):
+    lens = [1, 0, bs - 1, bs, bs + 1, 5 * bs + 3, 0, 301]
+    c = cases.make_case(300 + bs, lens, 64, block_size=bs, num_heads=32, num_kv_heads=4, cache=cache, pad=-1)
+    want = oracle_decode(c)
+    live = [i for i, n in enumerate(lens) if n > 0]
+    for kw in (dict(), dict(partition_size=48), dict(kv_heads_per_wave=2, partition_size=64)):
+        got = gpu_decode(pa, c, gpu, q_heads_per_wave=16, **kw)
+        check(got[live], want[live], cache)
+        assert float(got[[1, 6]].float().abs().max()) == 0.0       # rows without context come back as zeros
+
+
+@pytest.mark.parametrize("qdt", [torch.float32, torch.bfloat16, torch.float16])
+def test_matrix_kernel_query_dtypes_and_large_scores(pa, gpu, qdt):
+    """Scores far from zero (queries and keys of norm ~40): the reference point of the exponentials is
+    set by the first tile and moved when a later one outgrows it."""
+    c = cases.make_case(77, [700, 45, 2048, 9], 256, num_heads=32, num_kv_heads=8, q_dtype=qdt)
+    c["q"] = (c["q"].float() * 3.5).to(qdt)
+    # keys grow along the context, so later tiles hold the larger scores
+    ramp = torch.linspace(0.2, 3.0, c["k_cache"].shape[0] * c["k_cache"].shape[1]).view(c["k_cache"].shape[0], -1, 1, 1)
+    c["k_cache"] = (c["k_cache"].float() * ramp).to(c["k_cache"].dtype)
+    want = oracle_decode(c)
+    kind = "bf16" if qdt == torch.bfloat16 else "fp16"
+    check(gpu_decode(pa, c, gpu, q_heads_per_wave=16), want, kind)
+    check(gpu_decode(pa, c, gpu, q_heads_per_wave=16, partition_size=512, kv_heads_per_wave=2), want, kind)
+
+
+def test_matrix_kernel_is_the_choice_for_wide_groups(pa, gpu):
+    """From a ratio of 3 on the launch takes the matrix kernel by itself: same result as when it is
+    named, bit for bit, and the vector kernel agrees to rounding."""
+    c = cases.make_case(91, [500, 131, 64, 1999], 192, num_heads=24, num_kv_heads=8)
+    auto = gpu_decode(pa, c, gpu)
+    named = gpu_decode(pa, c, gpu, q_heads_per_wave=16)
+    vector = gpu_decode(pa, c, gpu, q_heads_per_wave=1)
+    assert torch.equal(auto, named)
+    torch.testing.assert_close(auto.float(), vector.float(), rtol=1e-3, atol=1e-3)
+    check(auto, oracle_decode(c), "fp16")
+
+
+def test_matrix_kernel_refuses_what_it_cannot_run(pa, gpu):
+    c = cases.make_case(5, [100, 50], 32, num_heads=28, num_kv_heads=7)
+    for kw in (dict(waves=1), dict(kv_heads_per_wave=2), dict(kv_heads_per_wave=4)):
+        with pytest.raises(RuntimeError, match="matrix path"):
+            gpu_decode(pa, c, gpu, q_heads_per_wave=16, **kw)
