@@ -17,8 +17,8 @@
 //    tile's loads are issued into the freed registers before the products start.
 //  * S^T = K . Q^T with v_mfma_f32_16x16x32_f16: A = 16 keys x 32 dims read back with
 //    ds_read_b128, B = Q^T (16 head columns, zero beyond the group) kept in registers, pre-scaled
-//    by scale*log2(e) and split into two fp16 parts (hi + lo, two products per step); the
-//    accumulator starts at -m_ref so exp2 applies directly to the result.
+//    by scale*log2(e) and, for 16-bit caches, split into two fp16 parts (hi + lo, two products per
+//    step); the accumulator starts at -m_ref so exp2 applies directly to the result.
 //  * O^T += V^T . P^T: A = 16 dims x 32 keys through the LDS transpose read ds_read_b64_tr_b16,
 //    B = P^T straight from the score registers (lane (head, g) holds keys 4g..4g+3 of both
 //    16-key halves; the products label the contraction index accordingly).
@@ -161,9 +161,11 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   if (begin >= end) return;
 
   // ---- Q^T as the B operand: lane (col, kg) holds dims 32c + 8kg .. +7 of head col, step c ----------
-  // in two fp16 parts, q * scale * log2(e) = hi + lo to 22 bits: the matrix pipe has time to spare,
-  // and a single fp16 rounding of the query costs 2^-12 of the score, visible where logits are large
-  mhalf8_t qreg[HPW][KSTEPS], qlo[HPW][KSTEPS];
+  // 16-bit caches: in two fp16 parts, q * scale * log2(e) = hi + lo to 22 bits.  The matrix pipe has
+  // time to spare, and a single fp16 rounding of the query costs 2^-12 of the score, visible where
+  // logits are large.  fp8 caches (tolerance 1e-2) take the one part.
+  constexpr bool SPLIT_Q = KV != KV_FP8;
+  mhalf8_t qreg[HPW][KSTEPS], qlo[SPLIT_Q ? HPW : 1][SPLIT_Q ? KSTEPS : 1];
   {
     const bool live = col < nh;
     auto load_q = [&](auto dt_tag) __attribute__((always_inline)) {
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
             const float qs = live ? x[e] * p.scale_log2e : 0.0f;
             const _Float16 hi = (_Float16)qs;
             qreg[hh][c][e] = hi;
-            qlo[hh][c][e] = (_Float16)(qs - (float)hi);
+            if constexpr (SPLIT_Q) qlo[hh][c][e] = (_Float16)(qs - (float)hi);
           }
         }
       }
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
         for (int kb = 0; kb < 2; ++kb) {
           const mhalf8_t a = *(const mhalf8_t*)(k_rd[c] + (hh * TILEB + kb * 16 * ROWB));
           s[hh][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qreg[hh][c], s[hh][kb], 0, 0, 0);
-          s2[hh][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qlo[hh][c], s2[hh][kb], 0, 0, 0);
+          if constexpr (SPLIT_Q) s2[hh][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qlo[hh][c], s2[hh][kb], 0, 0, 0);
         }
     const int lim = masked ? end - (begin + tile * TILE) : TILE;   // keys of the tile below this are real
     float mloc[HPW];
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float x = s[hh][kb][e] + s2[hh][kb][e];
+          const float x = SPLIT_Q ? s[hh][kb][e] + s2[hh][kb][e] : s[hh][kb][e];
           s[hh][kb][e] = (16 * kb + 4 * kg + e) < lim ? x : NEG_INF;
         }
       float mx = s[hh][0][0];

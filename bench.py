@@ -17,8 +17,8 @@ what the command line asked for; the launches actually timed are under `timing`.
 Prints ONE JSON line.  `roofline` is for the dominant kernel (the attention pass alone);
 `cpu_baseline` times the oracle (the reference's PyTorch fallback restated) on a bounded
 sample of the same workload.  `other_configs` holds the decode launches of BASELINE configs 1,
-3 and 4 (same recipe as the parity tests: seeds 1001 / 1003 / 1004) and of 32 and 64 query heads
-over the 8 KV heads at the headline batch and context.
+3 and 4 (same recipe as the parity tests: seeds 1001 / 1003 / 1004), `gqa_decode` those of 32 and
+64 query heads over the 8 KV heads at the headline batch and context, FP16 and FP8 KV.
 """
 import argparse
 import json
@@ -259,25 +259,11 @@ def other_decode_configs(pa, torch, dev, launches):
     meta["cfg4"] = dict(workload="32 prompts x 8 samples, shared 1024-token prefix, suffix U[64,512] (seed 1004), FP16 KV",
                         kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
-    # wider GQA groups at the headline batch and context: every KV row is still read once, by the
-    # one workgroup that serves all query heads of its KV head
-    gqa = {}
-    for name, hq in (("gqa4", 32), ("gqa8", 64)):
-        w, _ = _paged_case(torch, dev, [4096] * 64, 1100 + hq, hq=hq)
-        gqa[name] = w
-        fns[name] = lambda w=w: pa.paged_decode(w["q"], w["k_cache"], w["v_cache"], w["block_tables"],
-                                                w["context_lens"], scale, out=w["out"])
-        meta[name] = dict(workload="batch 64, ctx 4096, %d q / 8 kv heads (GQA %d), FP16 KV" % (hq, hq // 8),
-                          alg_bytes=algorithmic_bytes(64, 4096, hq, HKV, D, BS, False))
-
     t = time_alternating(torch, fns, launches)
     for name, m in meta.items():
         us = med(t[name])
         rec = {"workload": m["workload"], "us": spread(t[name])}
-        if "alg_bytes" in m:
-            rec.update(algorithmic_bytes=m["alg_bytes"], gbps=round(m["alg_bytes"] / us / 1e3, 1),
-                       frac_of_8TBps=round(m["alg_bytes"] / us / 1e3 / HBM_PEAK_GBPS, 4))
-        elif "note" in m:
+        if "note" in m:
             rec["note"] = m["note"]
             rec["kv_bytes"] = m["kv_bytes"]
         elif "unique_kv_bytes" in m:
@@ -292,6 +278,36 @@ def other_decode_configs(pa, torch, dev, launches):
                        partitions_launched=m["partitions_launched"], gbps=round(total / us / 1e3, 1),
                        frac_of_8TBps=round(total / us / 1e3 / HBM_PEAK_GBPS, 4))
         out[name] = rec
+    return out
+
+
+def gqa_decode_configs(pa, torch, dev, launches, which):
+    """Wider query groups at the headline batch and context (batch 64, ctx 4096, 8 KV heads x 128, block 16):
+    every KV row is read once, by the one workgroup that serves all query heads of its KV head; from a
+    ratio of 3 on the launch multiplies on the matrix cores.  `which`: entries like "4", "8fp8" = GQA
+    ratio and cache type.  The launches alternate in one timed loop."""
+    HKV, D, BS = 8, 128, 16
+    scale = D ** -0.5
+    fns, meta, keep = {}, {}, []
+    for item in which:
+        fp8 = item.endswith("fp8")
+        ratio = int(item[:-3] if fp8 else item)
+        hq = ratio * HKV
+        name = "gqa%d%s" % (ratio, "_fp8" if fp8 else "")
+        w = build_workload(pa, torch, dev, 64, 4096, hq, HKV, D, BS, fp8, 1100 + hq)
+        w["out"] = torch.empty_like(w["q"])
+        keep.append(w)
+        fns[name] = lambda w=w: pa.paged_decode(w["q"], w["k_cache"], w["v_cache"], w["block_tables"], w["context_lens"],
+                                                scale, w["k_scale"], w["v_scale"], out=w["out"])
+        meta[name] = dict(workload="batch 64, ctx 4096, %d q / 8 kv heads (GQA %d), %s KV" % (hq, ratio, "FP8" if fp8 else "FP16"),
+                          alg_bytes=algorithmic_bytes(64, 4096, hq, HKV, D, BS, fp8))
+    t = time_alternating(torch, fns, launches)
+    out = {}
+    for name, m in meta.items():
+        us = med(t[name])
+        out[name] = {"workload": m["workload"], "us": spread(t[name]), "algorithmic_bytes": m["alg_bytes"],
+                     "gbps": round(m["alg_bytes"] / us / 1e3, 1),
+                     "frac_of_8TBps": round(m["alg_bytes"] / us / 1e3 / HBM_PEAK_GBPS, 4)}
     return out
 
 
@@ -621,6 +637,17 @@ def model_step_cfg5b(pa, torch, dev, steps, warmup):
     return out
 
 
+def copy_calibration(torch, dev):
+    """Three plain 1 GiB device-to-device copies: known traffic for scaling FETCH_SIZE / WRITE_SIZE."""
+    src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -638,11 +665,14 @@ def main():
                     help="launches per timed repeat are max(steps, this); profiler runs with counters lower it")
     ap.add_argument("--sections", default="all",
                     help="comma-separated parts to run: headline (the FP16 / FP8 launches), probe (the same "
-                         "launches with loads only), others (configs 1, 3, 4 and the wider GQA groups), prefill, "
+                         "launches with loads only), others (configs 1, 3, 4), gqa (wider query groups), prefill, "
                          "extras, cpu; 'all' = every one.  For profiler runs, which want one kind of launch "
                          "per kernel name: the load probe is the decode kernel itself with a flag set, and the "
                          "other configurations launch the headline's kernels on other shapes.  Without "
                          "`headline` the run prints a reduced line for the parts it ran")
+    ap.add_argument("--gqa", default="4,8,4fp8,8fp8",
+                    help="the launches of the gqa section: GQA ratios over 8 KV heads, 'fp8' appended for an FP8 cache "
+                         "(a profiler run names one, so that the kernel name stands for one workload)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device-to-device copies (known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
@@ -655,12 +685,12 @@ def main():
 
     sections = set(args.sections.split(","))
     if "all" in sections:
-        sections = {"headline", "probe", "others", "prefill", "extras", "cpu"}
+        sections = {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}
     if args.no_extras:
         sections.discard("extras")
     if args.no_cpu_baseline:
         sections.discard("cpu")
-    unknown = sections - {"headline", "probe", "others", "prefill", "extras", "cpu"}
+    unknown = sections - {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}
     if unknown:
         print("bench.py: unknown section(s) %s" % sorted(unknown), file=sys.stderr)
         sys.exit(2)
@@ -672,8 +702,12 @@ def main():
         torch.cuda.set_device(dev)
         launches = max(args.steps, args.min_launches)
         part = {"sections": sorted(sections)}
+        if args.copy_calibration:
+            copy_calibration(torch, dev)
         if "others" in sections:
             part["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+        if "gqa" in sections:
+            part["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
         if "prefill" in sections:
             part["prefill_mfma"] = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup))
         print(json.dumps(part))
@@ -687,13 +721,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.copy_calibration:
-        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-        torch.cuda.empty_cache()
+        copy_calibration(torch, dev)
 
     B, CTX, HQ, HKV, D, BS = args.batch, args.ctx, 16, 8, 128, 16
     scale = 1.0 / math.sqrt(D)
@@ -856,6 +884,8 @@ def main():
         line["roofline"]["fp8_kernel"]["frac_of_plain_stream_read"] = round(f8["kernel_gbps"] / stream_read["best_gbps"], 4)
     if "others" in sections:
         line["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+    if "gqa" in sections:
+        line["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
     if prefill is not None:
         line["prefill_mfma"] = prefill
     if "extras" in sections:
