@@ -12,9 +12,10 @@
 //    token (256 bytes of fp8 instead of 128) and multiplies one head after the other.
 //  * Loads are those of the vector kernel: 16 bytes per lane, the 8 lanes of a token row read one
 //    contiguous piece, one register tile (32 tokens of K and of V) in flight per wave.
-//  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16, fp8
-//    times 1 / the token's scale) to the wave's own 2 x 32 x head_dim fp16 of LDS, and the next
-//    tile's loads are issued into the freed registers before the products start.
+//  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16; fp8 bytes
+//    are exact in fp16, their per-token scales go to LDS beside the tile and are applied to the
+//    scores and the probabilities after the products) to the wave's own 2 x 32 x head_dim fp16 of
+//    LDS, and the next tile's loads are issued into the freed registers before the products start.
 //  * S^T = K . Q^T with v_mfma_f32_16x16x32_f16: A = 16 keys x 32 dims read back with
 //    ds_read_b128, B = Q^T (16 head columns, zero beyond the group) kept in registers, pre-scaled
 //    by scale*log2(e) and, for 16-bit caches, split into two fp16 parts (hi + lo, two products per
@@ -50,8 +51,12 @@ __device__ __forceinline__ constexpr int lds_swz(int row) {
 
 // K and V tile of one KV head
 __host__ __device__ constexpr int decode_mfma_tile_bytes(int D) { return 2 * kMfmaTile * D * 2; }
+// per wave: its tiles, then 1 / scale of the tile's 32 tokens for K and for V (fp8 caches)
+__host__ __device__ constexpr int decode_mfma_wave_bytes(int HPW, int D) {
+  return HPW * decode_mfma_tile_bytes(D) + 2 * kMfmaTile * 4;
+}
 __host__ __device__ constexpr int decode_mfma_lds_bytes(int W, int HPW, int D) {
-  return W * HPW * decode_mfma_tile_bytes(D) + 2 * HPW * kMfmaHeads * W * 4;
+  return W * decode_mfma_wave_bytes(HPW, D) + 2 * HPW * kMfmaHeads * W * 4;
 }
 
 template <int KV, int D, int HPW>
@@ -66,7 +71,7 @@ struct MfmaTile {
 
 // 8 source elements (4 dwords of a 16-bit cache, 2 dwords of fp8) -> 8 fp16
 template <int KV>
-__device__ __forceinline__ mhalf8_t words_to_f16(const uint32_t* w, float inv_scale) {
+__device__ __forceinline__ mhalf8_t words_to_f16(const uint32_t* w) {
   mhalf8_t r;
   if constexpr (KV == KV_F16) {
     const uint32_t ww[4] = {w[0], w[1], w[2], w[3]};
@@ -78,16 +83,12 @@ __device__ __forceinline__ mhalf8_t words_to_f16(const uint32_t* w, float inv_sc
       r[2 * i + 1] = (_Float16)__uint_as_float(w[i] & 0xffff0000u);
     }
   } else {
-    // byte * inv_scale = byte * m * 2^e, m in [1, 2): the conversion applies 2^e exactly, the
-    // mantissa is one packed fp16 multiply per pair
-    const uint32_t bits = __float_as_uint(inv_scale);
-    const float pow2 = __uint_as_float(bits & 0xff800000u);
-    const _Float16 m = (_Float16)__uint_as_float((bits & 0x007fffffu) | 0x3f800000u);
-    const half2_t mm = {m, m};
+    // the bytes as they are (exact in fp16); the token's scale is applied to the score and to the
+    // probability after the products
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const half2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, false) * mm;
-      const half2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, true) * mm;
+      const half2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, false);
+      const half2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, true);
       r[4 * i] = lo[0];
       r[4 * i + 1] = lo[1];
       r[4 * i + 2] = hi[0];
@@ -119,9 +120,11 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   extern __shared__ __align__(16) uint8_t lds_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  uint8_t* my_lds = lds_raw + wave * HPW * TILEB;      // this wave's tiles: per KV head K, then V
+  constexpr int WAVEB = decode_mfma_wave_bytes(HPW, D);
+  uint8_t* my_lds = lds_raw + wave * WAVEB;            // this wave's tiles: per KV head K, then V
+  float* my_scales = reinterpret_cast<float*>(my_lds + HPW * TILEB);   // [2][TILE]: 1 / k_scale, 1 / v_scale per token
   float (*red)[HPW * NHC * D] = reinterpret_cast<float (*)[HPW * NHC * D]>(lds_raw);   // [W][HPW * NHC * D], over the tiles
-  float (*sm)[W] = reinterpret_cast<float (*)[W]>(lds_raw + W * HPW * TILEB);          // [HPW * NHC][W]
+  float (*sm)[W] = reinterpret_cast<float (*)[W]>(lds_raw + W * WAVEB);                // [HPW * NHC][W]
   float (*sl)[W] = sm + HPW * NHC;                                                      // [HPW * NHC][W]
 
   const int g = lane >> 3;        // row group of the loads
@@ -264,19 +267,14 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     for (int r = 0; r < RL; ++r) {
       const int tk = token_of(r);
       const bool valid = !masked || (begin + tile * TILE + tk) < end;
-      float iks = 1.0f, ivs = 1.0f;
-      if constexpr (KV == KV_FP8) {
-        iks = __builtin_amdgcn_rcpf(t.ks[r]);
-        ivs = __builtin_amdgcn_rcpf(t.vs[r]);
-      }
 #pragma unroll
       for (int c = 0; c < G::NLD; ++c) {
 #pragma unroll
         for (int x = 0; x < CPL; ++x) {
           const int chunk = (c * 8 + j) * CPL + x;
           const int wpc = (KV == KV_FP8) ? 2 : 4;   // dwords per 8 source elements
-          mhalf8_t kf = words_to_f16<KV>(&t.k[r][c * (G::LB / 4) + x * wpc], iks);
-          mhalf8_t vf = words_to_f16<KV>(&t.v[r][c * (G::LB / 4) + x * wpc], ivs);
+          mhalf8_t kf = words_to_f16<KV>(&t.k[r][c * (G::LB / 4) + x * wpc]);
+          mhalf8_t vf = words_to_f16<KV>(&t.v[r][c * (G::LB / 4) + x * wpc]);
           if (!valid) {
             // rows past the end: their scores are masked, and their V must not turn 0 * garbage into NaN
 #pragma unroll
@@ -286,6 +284,23 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
           *(mhalf8_t*)dst = kf;
           *(mhalf8_t*)(dst + TILE * ROWB) = vf;
         }
+      }
+    }
+    if constexpr (KV == KV_FP8) {
+      // 1 / scale per token, 0 for rows past the end (their V rows are zero, and 0 * 0 stays 0).  The 8
+      // lanes of a row group (and both heads' groups) hold the same values and write the same words.
+#pragma unroll
+      for (int sb = 0; sb < NSUB; ++sb) {
+        float ik[4], iv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const bool valid = !masked || (begin + tile * TILE + token_of(4 * sb + r)) < end;
+          ik[r] = valid ? __builtin_amdgcn_rcpf(t.ks[4 * sb + r]) : 0.0f;
+          iv[r] = valid ? __builtin_amdgcn_rcpf(t.vs[4 * sb + r]) : 0.0f;
+        }
+        const int tok0 = token_of(4 * sb);
+        *(float4*)&my_scales[tok0] = make_float4(ik[0], ik[1], ik[2], ik[3]);
+        *(float4*)&my_scales[TILE + tok0] = make_float4(iv[0], iv[1], iv[2], iv[3]);
       }
     }
   };
@@ -326,11 +341,22 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     mfloat4_t s[HPW][2], s2[HPW][2];
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
-      const float nr = -m_ref[hh];
+      const float nr = KV == KV_FP8 ? 0.0f : -m_ref[hh];   // fp8: the scale comes first, the reference after it
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         s[hh][kb] = mfloat4_t{nr, nr, nr, nr};
         s2[hh][kb] = mfloat4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+    }
+    // fp8: 1 / scale of this lane's 8 keys (4kg .. 4kg+3 of both halves)
+    float iks[2][4], ivs[2][4];
+    if constexpr (KV == KV_FP8) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const float4 a = *(const float4*)&my_scales[16 * kb + 4 * kg];
+        const float4 b2 = *(const float4*)&my_scales[TILE + 16 * kb + 4 * kg];
+        iks[kb][0] = a.x; iks[kb][1] = a.y; iks[kb][2] = a.z; iks[kb][3] = a.w;
+        ivs[kb][0] = b2.x; ivs[kb][1] = b2.y; ivs[kb][2] = b2.z; ivs[kb][3] = b2.w;
       }
     }
 #pragma unroll
@@ -352,7 +378,9 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float x = SPLIT_Q ? s[hh][kb][e] + s2[hh][kb][e] : s[hh][kb][e];
+          float x;
+          if constexpr (KV == KV_FP8) x = fmaf(s[hh][kb][e], iks[kb][e], -m_ref[hh]);
+          else x = SPLIT_Q ? s[hh][kb][e] + s2[hh][kb][e] : s[hh][kb][e];
           s[hh][kb][e] = (16 * kb + 4 * kg + e) < lim ? x : NEG_INF;
         }
       float mx = s[hh][0][0];
@@ -395,10 +423,18 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
-          const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
-          psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
-          pb[hh][4 * kb + e] = h[0];
-          pb[hh][4 * kb + e + 1] = h[1];
+          if constexpr (KV == KV_FP8) {
+            // the row sum takes the probability, the product the probability / v_scale
+            const float p0 = __builtin_amdgcn_exp2f(s[hh][kb][e]), p1 = __builtin_amdgcn_exp2f(s[hh][kb][e + 1]);
+            psum += p0 + p1;
+            pb[hh][4 * kb + e] = (_Float16)(p0 * ivs[kb][e]);
+            pb[hh][4 * kb + e + 1] = (_Float16)(p1 * ivs[kb][e + 1]);
+          } else {
+            const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
+            psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
+            pb[hh][4 * kb + e] = h[0];
+            pb[hh][4 * kb + e + 1] = h[1];
+          }
         }
       l_run[hh] += psum;
     }

@@ -430,3 +430,38 @@ def test_matrix_kernel_refuses_what_it_cannot_run(pa, gpu):
     for kw in (dict(waves=1), dict(kv_heads_per_wave=2), dict(kv_heads_per_wave=4)):
         with pytest.raises(RuntimeError, match="matrix path"):
             gpu_decode(pa, c, gpu, q_heads_per_wave=16, **kw)
+
+
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_matrix_kernel_in_a_replayed_graph(pa, gpu, cache):
+    """Single pass and partitioned launches of the matrix kernel recorded in one graph; every replay,
+    with eager work and new context lengths between the replays, equals the eager result."""
+    lens = [900, 31, 1500, 257]
+    c = cases.make_case(123, lens, 192, num_heads=32, num_kv_heads=4, cache=cache)
+    d = cases.to_device(c, gpu)
+    out1, out2 = torch.empty_like(d["q"]), torch.empty_like(d["q"])
+
+    def run():
+        pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"], d["scale"],
+                        d["k_scale"], d["v_scale"], out=out1)
+        pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"], d["scale"],
+                        d["k_scale"], d["v_scale"], partition_size=256, out=out2)
+
+    run()                                         # eager warm-up: workspace and kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    torch.cuda.synchronize()
+    for shrink in (0, 100, 7):
+        new_lens = [n - min(shrink, n - 1) for n in lens]
+        d["context_lens"].copy_(torch.tensor(new_lens, dtype=torch.int32))
+        c["context_lens"] = torch.tensor(new_lens, dtype=torch.int32)
+        want = oracle_decode(c)
+        out1.fill_(float("nan"))
+        out2.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        check(out1.cpu(), want, cache)
+        check(out2.cpu(), want, cache)
+        _ = torch.randn(1 << 16, device=gpu).sum().item()      # eager work between the replays
