@@ -37,6 +37,10 @@ SIGNATURES = {
     "pa_decode": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr, _ptr,
                          _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
                          _int, _int, _int, _ptr]),
+    "pa_decode_shared_prefix": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr, _ptr,
+                                       _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
+                                       _int, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
+    "pa_check_shared_prefix": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
     "pa_decode_noalloc": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
                                  _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64,
                                  _int, _int, _int, _ptr]),

@@ -553,6 +553,150 @@ def choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, k
     return psize, parts, 0
 
 
+# ---- shared prefixes ---------------------------------------------------------------------------
+SHARED_PREFIX_PARTITION = 256      # tokens; the granularity at which a shared prefix is computed once
+
+
+def find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads,
+                       partition_size=SHARED_PREFIX_PARTITION):
+    """Host-side: runs of consecutive rows whose leading table entries name the same physical
+    blocks (n samples of a prompt, forks of a cached prefix), as [(first_row, rows, shared_tokens)].
+    block_tables: per-row lists of block ids (what the cache manager holds on the host);
+    context_lens: per-row token counts.  Only whole partitions count, a group needs two rows and
+    one shared partition, and holds at most 16 // (num_q_heads // num_kv_heads) rows (the columns
+    of the matrix kernel's operand); longer runs are cut into several groups, and a run ends where
+    the next row would shrink what the group shares by more than it adds."""
+    max_rows = 16 // max(1, num_q_heads // num_kv_heads)
+    if max_rows < 2:
+        return []
+    part_blocks = partition_size // block_size
+    groups, n, b = [], len(block_tables), 0
+    while b < n:
+        lead = block_tables[b]
+        limit = min(len(lead), int(context_lens[b]) // block_size)     # whole blocks inside the context
+        rows, shared = 1, limit
+        while b + rows < n and rows < max_rows:
+            other = block_tables[b + rows]
+            cap = min(shared, len(other), int(context_lens[b + rows]) // block_size)
+            common = 0
+            while common < cap and other[common] == lead[common]:
+                common += 1
+            # a group of n rows saves n - 1 reads of its shared partitions: stop where taking the row
+            # in would shrink the shared part by more than that adds
+            new_parts, old_parts = common // part_blocks, shared // part_blocks
+            if new_parts < 1 or (new_parts < old_parts and rows * new_parts <= (rows - 1) * old_parts):
+                break
+            shared = common
+            rows += 1
+        if rows >= 2:
+            groups.append((b, rows, (shared // part_blocks) * partition_size))
+        b += rows
+    return groups
+
+
+def shared_prefix_descriptors(groups, batch, device, partition_size=SHARED_PREFIX_PARTITION):
+    """Device descriptors of a pa_decode_shared_prefix launch from [(first_row, rows, shared_tokens)]:
+    (group_desc int32 [G, 4], row_skip int32 [batch], most rows per group, most shared partitions,
+    fewest partitions any row skips)."""
+    desc = torch.zeros((max(len(groups), 1), 4), dtype=torch.int32)
+    skip = torch.zeros(batch, dtype=torch.int32)
+    max_rows = max_parts = 0
+    for i, (first, rows, shared_tokens) in enumerate(groups):
+        parts = int(shared_tokens) // partition_size
+        if first < 0 or rows < 1 or first + rows > batch:
+            raise RuntimeError("shared_prefix_descriptors: group (%d, %d) reaches outside the batch of %d" % (first, rows, batch))
+        desc[i, 0], desc[i, 1], desc[i, 2] = first, rows, parts
+        skip[first:first + rows] = parts
+        max_rows, max_parts = max(max_rows, rows), max(max_parts, parts)
+    min_skip = int(skip.min()) if batch else 0
+    return desc.to(device), skip.to(device), max_rows, max_parts, min_skip
+
+
+def prepare_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, device,
+                          partition_size=2 * SHARED_PREFIX_PARTITION):
+    """What a decode step hands the attention layers (InferenceContext.prefix_groups) when rows share
+    prefixes: the groups found on the host in the per-row block-id lists and their device descriptors,
+    built once per step for all layers.  None when no two rows share a whole partition."""
+    groups = find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, partition_size)
+    if not groups:
+        return None
+    return {"groups": groups, "partition_size": int(partition_size),
+            "descriptors": shared_prefix_descriptors(groups, len(block_tables), device, partition_size)}
+
+
+def paged_decode_shared_prefix(q, k_cache, v_cache, block_tables, context_lens, scale, groups, k_scale=None,
+                               v_scale=None, partition_size=SHARED_PREFIX_PARTITION, out=None, waves=0,
+                               workspace=None, descriptors=None):
+    """paged_decode for a batch with shared prefixes: `groups` = [(first_row, rows, shared_tokens)]
+    (find_prefix_groups), or `descriptors` = what shared_prefix_descriptors returned for them (to
+    keep the host-to-device copies out of a step).  Partitions inside a group's shared prefix are
+    read once per group.  Same result as paged_decode(partition_size=partition_size).  The groups
+    are trusted; PA_DEBUG_TABLES=1 checks them against the tables before every launch."""
+    _require_gpu(q, "paged_decode_shared_prefix")
+    _require_gpu(k_cache, "paged_decode_shared_prefix")
+    _check_cache(k_cache, v_cache, "paged_decode_shared_prefix")
+    lib = _native.load()
+    if q.dim() != 3:
+        raise RuntimeError("paged_decode_shared_prefix: q must be [batch, heads, head_dim]")
+    batch, num_q_heads, head_dim = q.shape
+    num_blocks, block_size, num_kv_heads, d2 = k_cache.shape
+    if d2 != head_dim:
+        raise RuntimeError("paged_decode_shared_prefix: q head_dim %d != cache head_dim %d" % (head_dim, d2))
+    if block_tables.dim() != 2 or block_tables.shape[0] != batch or context_lens.numel() != batch:
+        raise RuntimeError("paged_decode_shared_prefix: block_tables/context_lens do not match the batch")
+    psize = int(partition_size)
+    if psize <= 0 or psize % 16 or psize % block_size:
+        raise RuntimeError("paged_decode_shared_prefix: partition_size must be a multiple of 16 and of the block size")
+    q, qs = _rows(q, "paged_decode_shared_prefix")
+    tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
+    if tables.stride(1) != 1:
+        tables = tables.contiguous()
+    lens = _int32(context_lens, "paged_decode_shared_prefix")
+    if out is None:
+        out = torch.empty((batch, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+    if batch == 0:
+        return out
+    kv_code = _code(k_cache.dtype, "paged_decode_shared_prefix")
+    fp8 = kv_code == _native.DTYPE_FP8_E4M3
+    if fp8 and (k_scale is None or v_scale is None):
+        raise RuntimeError("paged_decode_shared_prefix: fp8 cache needs k_scale and v_scale")
+    if descriptors is None:
+        descriptors = shared_prefix_descriptors(groups, batch, q.device, psize)
+        num_groups = len(groups)
+    else:
+        num_groups = len(groups) if groups is not None else descriptors[0].shape[0]
+    desc, skip, max_rows, max_shared, min_skip = descriptors
+    parts = max(1, (tables.shape[1] * block_size + psize - 1) // psize)
+    if _debug_tables():
+        counts = torch.zeros(3, dtype=torch.int32, device=q.device)
+        rc = lib.pa_check_shared_prefix(tables.data_ptr(), tables.stride(0), tables.shape[1], lens.data_ptr(), batch,
+                                        block_size, psize, desc.data_ptr(), num_groups, skip.data_ptr(),
+                                        counts.data_ptr(), _stream_ptr(q.device))
+        _native.check(rc, "pa_check_shared_prefix")
+        differ, short, stray = counts.tolist()
+        if differ or short or stray:
+            raise RuntimeError("paged_decode_shared_prefix: %d shared table entries differ inside their group, %d rows "
+                               "too short for their group or with the wrong row_skip, %d rows outside the groups "
+                               "with a row_skip or inside two groups" % (differ, short, stray))
+    ws_bytes = lib.pa_workspace_bytes(batch, num_q_heads, head_dim, parts)
+    if workspace is not None:
+        if workspace.dtype != torch.uint8 or not workspace.is_cuda or workspace.numel() < ws_bytes:
+            raise RuntimeError("paged_decode_shared_prefix: workspace must be a uint8 GPU tensor of at least %d bytes" % ws_bytes)
+        ws = workspace
+    else:
+        ws = reserve_decode_workspace(q.device, ws_bytes)
+    own = max(1, parts - min_skip)      # every row computes what its group does not
+    rc = lib.pa_decode_shared_prefix(q.data_ptr(), _code(q.dtype, "paged_decode_shared_prefix"), qs, k_cache.data_ptr(),
+                                     v_cache.data_ptr(), k_scale.data_ptr() if fp8 else None,
+                                     v_scale.data_ptr() if fp8 else None, kv_code, tables.data_ptr(),
+                                     tables.stride(0), tables.shape[1], lens.data_ptr(), out.data_ptr(), out.stride(0),
+                                     batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, float(scale),
+                                     psize, parts, ws.data_ptr(), ws_bytes, int(waves or 0), desc.data_ptr(), num_groups,
+                                     max(1, max_rows), max_shared, skip.data_ptr(), own, _stream_ptr(q.device))
+    _native.check(rc, "pa_decode_shared_prefix")
+    return out
+
+
 def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale=None,
                  v_scale=None, partition_size=None, out=None, waves=0, kv_heads_per_wave=None,
                  q_heads_per_wave=0, workspace=None):
@@ -758,8 +902,21 @@ class PagedAttention(nn.Module):
         if self.k_cache is None or ctx.block_tables is None or ctx.context_lens is None:
             return q  # nothing bound: same last-resort behaviour as attention.py:329-330
         ks, vs = self._scales()
+        shared = self._shared_prefix_decode(q, ctx, ks, vs)
+        if shared is not None:
+            return shared
         return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
                             self.scale, k_scale=ks, v_scale=vs)
+
+    def _shared_prefix_decode(self, q, ctx, ks, vs):
+        """Rows that share prefixes (ctx.prefix_groups, set by the runner when it found any): the shared
+        partitions are read once per group.  None when the step has no groups."""
+        pg = getattr(ctx, "prefix_groups", None)
+        if not pg or q.shape[0] != pg["descriptors"][1].numel():
+            return None
+        return paged_decode_shared_prefix(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
+                                          self.scale, pg["groups"], k_scale=ks, v_scale=vs,
+                                          partition_size=pg["partition_size"], descriptors=pg["descriptors"])
 
 
 class PartitionedPagedAttention(PagedAttention):
@@ -791,6 +948,9 @@ class PartitionedPagedAttention(PagedAttention):
         if self.k_cache is None or ctx.block_tables is None or ctx.context_lens is None:
             return q
         ks, vs = self._scales()
+        shared = self._shared_prefix_decode(q, ctx, ks, vs)
+        if shared is not None:
+            return shared
         psize = self.partition_size
         if self.adaptive:
             max_context = ctx.block_tables.shape[1] * self.k_cache.shape[1]

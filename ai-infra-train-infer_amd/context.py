@@ -26,6 +26,9 @@ class InferenceContext:
     context_lens: Optional[torch.Tensor] = None
     # [num_seqs, max_blocks] physical block ids; entries past the context are never read
     block_tables: Optional[torch.Tensor] = None
+    # decode, optional (no counterpart in the reference): rows that share prefixes as the same
+    # physical blocks, as attention.prepare_prefix_groups() returns them; None = read every row alone
+    prefix_groups: Optional[dict] = None
 
 
 _CONTEXT = InferenceContext()
@@ -40,6 +43,7 @@ def set_context(
     slot_mapping: Optional[torch.Tensor] = None,
     context_lens: Optional[torch.Tensor] = None,
     block_tables: Optional[torch.Tensor] = None,
+    prefix_groups: Optional[dict] = None,
 ):
     """Install the context for the next model forward."""
     global _CONTEXT
@@ -52,6 +56,7 @@ def set_context(
         slot_mapping=slot_mapping,
         context_lens=context_lens,
         block_tables=block_tables,
+        prefix_groups=prefix_groups,
     )
 
 

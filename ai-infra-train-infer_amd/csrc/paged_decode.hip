@@ -59,6 +59,43 @@ __global__ void check_tables_kernel(const int32_t* __restrict__ block_tables, in
   if (id < 0 || id >= num_blocks) atomicAdd(&counts[0], 1);
 }
 
+// Debug aid for shared-prefix launches: counts[0] = table entries of a group's shared partitions
+// that differ between a row and the group's first row; counts[1] = rows whose context is shorter
+// than the tokens their group shares, or whose row_skip differs from their group's shared
+// partitions; counts[2] = rows that belong to no group but have a non-zero row_skip, or to two groups.
+// One workgroup per group, one thread per shared table entry (strided).
+__global__ void check_shared_prefix_kernel(const int32_t* __restrict__ block_tables, int64_t bt_stride,
+                                           int table_width, const int32_t* __restrict__ context_lens,
+                                           int batch, int bs_log2, int partition_size,
+                                           const int32_t* __restrict__ group_desc, int num_groups,
+                                           const int32_t* __restrict__ row_skip, int32_t* counts) {
+  const int gi = blockIdx.x;
+  if (gi == num_groups) {
+    // rows outside every group must skip nothing; rows inside exactly one
+    for (int b = threadIdx.x; b < batch; b += blockDim.x) {
+      int owners = 0;
+      for (int k = 0; k < num_groups; ++k)
+        owners += (b >= group_desc[4 * k] && b < group_desc[4 * k] + group_desc[4 * k + 1]) ? 1 : 0;
+      if ((owners == 0 && row_skip[b] != 0) || owners > 1) atomicAdd(&counts[2], 1);
+    }
+    return;
+  }
+  const int first = group_desc[4 * gi], rows = group_desc[4 * gi + 1], parts = group_desc[4 * gi + 2];
+  const int shared_tokens = parts * partition_size;
+  const int shared_blocks = (shared_tokens + (1 << bs_log2) - 1) >> bs_log2;
+  if (first < 0 || rows < 1 || first + rows > batch || parts < 0) {
+    if (threadIdx.x == 0) atomicAdd(&counts[1], 1);
+    return;
+  }
+  for (int m = threadIdx.x; m < rows; m += blockDim.x)
+    if (context_lens[first + m] < shared_tokens || row_skip[first + m] != parts) atomicAdd(&counts[1], 1);
+  for (int e = threadIdx.x; e < shared_blocks * (rows - 1); e += blockDim.x) {
+    const int m = 1 + e / shared_blocks, c = e % shared_blocks;
+    if (c >= table_width || block_tables[(first + m) * bt_stride + c] != block_tables[first * bt_stride + c])
+      atomicAdd(&counts[0], 1);
+  }
+}
+
 // CUs of the current device (per device, asked once).
 static int compute_units() {
   static int cached[kMaxDevices] = {0};
@@ -136,6 +173,16 @@ static int scratch_for_current_device(void** out) {
 
 enum { kDecodeFull = 0, kDecodePartials = 1, kDecodeProbe = 2 };
 
+// What pa_decode_shared_prefix adds to a partitioned launch.
+struct SharedPrefix {
+  const int32_t* group_desc;
+  int64_t num_groups;
+  int64_t max_group_rows;
+  int64_t max_shared_partitions;
+  const int32_t* row_skip;
+  int64_t max_own_partitions;
+};
+
 constexpr int kMatrixPath = 16;            // q_heads_per_wave value that names the MFMA kernel
 constexpr int kMatrixPathFromRatio = 3;     // GQA ratio from which the automatic choice takes it
 
@@ -149,7 +196,7 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
                        int64_t num_blocks, float scale, int64_t partition_size,
                        int64_t max_partitions, void* workspace, int64_t workspace_bytes,
                        int waves, int kv_heads_per_wave, int q_heads_per_wave, int mode,
-                       void* stream) {
+                       void* stream, const SharedPrefix* shared = nullptr) {
   const bool merge = mode == kDecodeFull;
   char msg[256];
 #define PA_FAIL(code, text)                         \
@@ -200,9 +247,21 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   if (q_heads_per_wave != 0 && q_heads_per_wave != 1 && q_heads_per_wave != 2 && q_heads_per_wave != 4 &&
       q_heads_per_wave != kMatrixPath)
     PA_FAIL(PA_ERR_BAD_ARG, "q_heads_per_wave must be 0 (automatic), 1, 2, 4 or 16 (the matrix path)");
-  const bool direct = merge && max_partitions == 1;
+  const bool direct = merge && max_partitions == 1 && !shared;
+  if (shared) {
+    if (!shared->group_desc || !shared->row_skip) PA_FAIL(PA_ERR_BAD_ARG, "null group descriptors");
+    if (shared->num_groups < 0 || shared->num_groups > 0x7fffffff || shared->max_group_rows < 1 ||
+        shared->max_shared_partitions < 0 || shared->max_shared_partitions > max_partitions ||
+        shared->max_own_partitions < 1 || shared->max_own_partitions > max_partitions)
+      PA_FAIL(PA_ERR_BAD_ARG, "group counts out of range");
+    if (partition_size <= 0) PA_FAIL(PA_ERR_BAD_ARG, "a shared-prefix launch is a partitioned launch: partition_size > 0");
+    if ((num_q_heads / num_kv_heads) * shared->max_group_rows > kMatrixPath)
+      PA_FAIL(PA_ERR_UNSUPPORTED, "rows per group x query heads per KV head must not exceed 16");
+    if (kv_heads_per_wave > 1 || (q_heads_per_wave != 0 && q_heads_per_wave != kMatrixPath) || waves == 1)
+      PA_FAIL(PA_ERR_UNSUPPORTED, "a shared-prefix launch runs on the matrix path with one KV head per wave");
+  }
   if (!direct) {
-    if (max_partitions > 1 && (partition_size <= 0 || partition_size % 16 != 0))
+    if ((max_partitions > 1 || shared) && (partition_size <= 0 || partition_size % 16 != 0))
       PA_FAIL(PA_ERR_UNSUPPORTED, "partition_size must be a positive multiple of 16");
     const int64_t need = ws_bytes(batch, num_q_heads, head_dim, max_partitions);
     if (!workspace || workspace_bytes < need) PA_FAIL(PA_ERR_WORKSPACE, "workspace missing or too small");
@@ -223,7 +282,7 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   // MFMA operand: the choice from a GQA ratio of 3 on, where the vector kernel's arithmetic per
   // loaded byte starts to cost more than the loads (batch 64 x 4096 tokens, fp16 / fp8 cache: ratio 4
   // 187 / 103 us against 195 / 142 us, ratio 8 187 / 103 against 239 / 257, ratio 2 182 / 100.5 against 179 / 100).
-  bool matrix = q_heads_per_wave == kMatrixPath;
+  bool matrix = q_heads_per_wave == kMatrixPath || shared != nullptr;
   if (q_heads_per_wave == 0 && g >= kMatrixPathFromRatio && mode != kDecodeProbe && kv_heads_per_wave <= 2 &&
       (waves == 0 || waves >= 2) && !(kv_heads_per_wave == 2 && (waves == 8 || num_kv_heads % 2 != 0)))
     matrix = true;
@@ -245,7 +304,7 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
       s.waves = waves;
     } else {
       const int64_t wgs = (num_kv_heads / s.hpw) * slices * max_partitions * batch;
-      s.waves = (s.hpw == 1 && wgs < compute_units()) ? 8 : 4;
+      s.waves = (s.hpw == 1 && wgs < compute_units() && !shared) ? 8 : 4;
     }
   } else {
     if (q_heads_per_wave != 0) {
@@ -315,7 +374,23 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   hipStream_t st = (hipStream_t)stream;
   p.inner = (int)(num_kv_heads / s.hpw) * slices;
   p.probe = mode == kDecodeProbe ? 1 : 0;
-  const int64_t wgs = batch * max_partitions * p.inner;
+  p.group_desc = nullptr;
+  p.row_skip = nullptr;
+  p.num_prefix_wgs = p.prefix_parts = p.suffix_parts = 0;
+  int64_t wgs = batch * max_partitions * p.inner;
+  if (shared) {
+    const int64_t prefix_wgs = shared->num_groups * shared->max_shared_partitions * p.inner;
+    wgs = prefix_wgs + batch * shared->max_own_partitions * p.inner;
+    if (prefix_wgs > 0x7fffffff) {
+      snprintf(msg, sizeof(msg), "%s: too many workgroups for one launch", who);
+      return fail(PA_ERR_UNSUPPORTED, msg);
+    }
+    p.group_desc = shared->group_desc;
+    p.row_skip = shared->row_skip;
+    p.num_prefix_wgs = (int)prefix_wgs;
+    p.prefix_parts = (int)shared->max_shared_partitions;
+    p.suffix_parts = (int)shared->max_own_partitions;
+  }
   if (wgs > 0x7fffffff) {
     snprintf(msg, sizeof(msg), "%s: too many workgroups for one launch", who);
     return fail(PA_ERR_UNSUPPORTED, msg);
@@ -414,6 +489,48 @@ extern "C" int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_st
                      0, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale,
                      partition_size, max_partitions, workspace, workspace_bytes,
                      waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodePartials, stream);
+}
+
+extern "C" int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+                                       const void* v_cache, const float* k_scale, const float* v_scale,
+                                       int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
+                                       int64_t table_width, const int32_t* context_lens, void* out,
+                                       int64_t out_token_stride, int64_t batch, int64_t num_q_heads,
+                                       int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                       int64_t num_blocks, float scale, int64_t partition_size,
+                                       int64_t max_partitions, void* workspace, int64_t workspace_bytes,
+                                       int waves_per_workgroup, const int32_t* group_desc,
+                                       int64_t num_groups, int64_t max_group_rows,
+                                       int64_t max_shared_partitions, const int32_t* row_skip,
+                                       int64_t max_own_partitions, void* stream) {
+  const SharedPrefix sp = {group_desc, num_groups, max_group_rows, max_shared_partitions, row_skip,
+                           max_own_partitions};
+  return decode_impl("pa_decode_shared_prefix", q, q_dtype, q_token_stride, k_cache, v_cache, k_scale,
+                     v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, out,
+                     out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
+                     num_blocks, scale, partition_size, max_partitions, workspace, workspace_bytes,
+                     waves_per_workgroup, 0, 0, kDecodeFull, stream, &sp);
+}
+
+extern "C" int pa_check_shared_prefix(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
+                                      const int32_t* context_lens, int64_t batch, int64_t block_size,
+                                      int64_t partition_size, const int32_t* group_desc,
+                                      int64_t num_groups, const int32_t* row_skip, int32_t* counts,
+                                      void* stream) {
+  if (batch < 0 || bt_stride < 0 || table_width < 0 || num_groups < 0 || partition_size <= 0)
+    return fail(PA_ERR_BAD_ARG, "pa_check_shared_prefix: negative or zero size");
+  if (!counts) return fail(PA_ERR_BAD_ARG, "pa_check_shared_prefix: null pointer");
+  const int bs_log2 = ilog2_exact(block_size);
+  if (bs_log2 < 0) return fail(PA_ERR_UNSUPPORTED, "pa_check_shared_prefix: block_size must be a power of two");
+  if (batch == 0) return PA_OK;
+  if (!block_tables || !context_lens || !row_skip || (num_groups > 0 && !group_desc))
+    return fail(PA_ERR_BAD_ARG, "pa_check_shared_prefix: null pointer");
+  if (batch > 0x7fffffff || table_width > 0x7fffffff || num_groups >= 0x7fffffff || partition_size > 0x7fffffff)
+    return fail(PA_ERR_UNSUPPORTED, "pa_check_shared_prefix: batch, table or group count too large for one launch");
+  hipLaunchKernelGGL(check_shared_prefix_kernel, dim3((unsigned)num_groups + 1), dim3(256), 0,
+                     (hipStream_t)stream, block_tables, bt_stride, (int)table_width, context_lens,
+                     (int)batch, bs_log2, (int)partition_size, group_desc, (int)num_groups, row_skip, counts);
+  return check_launch("pa_check_shared_prefix");
 }
 
 extern "C" int pa_merge(const void* workspace, int64_t workspace_bytes, const int32_t* context_lens,

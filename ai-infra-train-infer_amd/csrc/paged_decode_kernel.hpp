@@ -66,6 +66,16 @@ struct DecodeParams {
   int inner;        // workgroups per (batch row, partition): KV head groups x slices of the query group
   int probe;        // 1: loads only, the arithmetic replaced by a checksum (pa_decode_load_probe)
   float scale_log2e;
+  // Shared prefixes (matrix kernel only; group_desc == nullptr: off).  Rows come in groups of
+  // consecutive batch rows whose first `shared partitions` x partition_size tokens are the same
+  // physical blocks: those partitions are computed once per group, by the first num_prefix_wgs
+  // workgroups, for all the group's rows at once; the other workgroups take every row's own
+  // partitions from row_skip[row] on.
+  const int32_t* group_desc;   // [groups][4]: first row, rows, shared partitions, unused
+  const int32_t* row_skip;     // [batch]: leading partitions of the row that its group computes
+  int num_prefix_wgs;          // groups x prefix_parts x inner
+  int prefix_parts;            // most shared partitions of any group
+  int suffix_parts;            // most own partitions of any row
 };
 
 // How a launch is cut: all fields are template parameters of the kernel it selects.

@@ -23,6 +23,9 @@
 //  * O^T += V^T . P^T: A = 16 dims x 32 keys through the LDS transpose read ds_read_b64_tr_b16,
 //    B = P^T straight from the score registers (lane (head, g) holds keys 4g..4g+3 of both
 //    16-key halves; the products label the contraction index accordingly).
+//  * Shared prefixes (DecodeParams::group_desc): the columns of the operand can also be the query
+//    heads of several batch rows, for partitions whose tokens those rows share as the same physical
+//    blocks - read once for the group instead of once per row.
 //  * The reference maximum m_ref is shared by the 4 lanes of a head column and only moves when a
 //    tile's maximum outgrows it by more than 2^8; the waves' partial results are merged through
 //    LDS at the end exactly as in the vector kernel.
@@ -134,17 +137,45 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   const int col = lane & 15;      // matrix layouts: head column / key row / dim row
   const int kg = lane >> 4;       // matrix layouts: group of 8 contraction indices, or of 4 result rows
 
-  const int in = blockIdx.x % p.inner;
-  const int u = blockIdx.x / p.inner;
-  const int part = u % p.max_partitions;
-  const int b = u / p.max_partitions;
+  // ---- which rows, KV heads and tokens this workgroup takes ------------------------------------------------
   const int gq = p.num_q_heads / p.num_kv_heads;
   const int kv_groups = p.num_kv_heads / HPW;
+  int b, part, in;
+  int members = 1;          // batch rows served at once: > 1 only for the shared partitions of a group
+  if (p.group_desc) {
+    int x = blockIdx.x;
+    if (x < p.num_prefix_wgs) {
+      in = x % p.inner;
+      const int u = x / p.inner;
+      part = u % p.prefix_parts;
+      const int32_t* desc = p.group_desc + 4 * (u / p.prefix_parts);
+      if (part >= desc[2]) return;
+      b = desc[0];
+      members = desc[1];
+    } else {
+      x -= p.num_prefix_wgs;
+      in = x % p.inner;
+      const int u = x / p.inner;
+      b = u / p.suffix_parts;
+      part = p.row_skip[b] + u % p.suffix_parts;
+      if (part >= p.max_partitions) return;
+    }
+  } else {
+    in = blockIdx.x % p.inner;
+    const int u = blockIdx.x / p.inner;
+    part = u % p.max_partitions;
+    b = u / p.max_partitions;
+  }
   const int kvg = in % kv_groups;
   const int sub = in / kv_groups;
-  const int nh = min(gq - sub * NHC, NHC);           // query heads per KV head in this workgroup
   const int kvh0 = kvg * HPW;                        // first KV head of the workgroup
+  // Columns of the matrix operand.  One row: query heads sub * 16 ... of the KV head.  A group's
+  // shared partition: column c = query head c % gq of row b + c / gq (gq * members <= 16).
+  const int cdiv = members > 1 ? gq : NHC + 1;
+  const int nh = members > 1 ? members * gq : min(gq - sub * NHC, NHC);   // live columns per KV head
   auto first_head = [&](int hh) { return (kvh0 + hh) * gq + sub * NHC; };   // first query head behind KV head kvh0 + hh
+  auto col_row = [&](int c) { return b + c / cdiv; };
+  auto col_head = [&](int hh, int c) { return first_head(hh) + c % cdiv; };
 
   const int ctx = p.context_lens[b];
   if (ctx <= 0) {
@@ -174,7 +205,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     auto load_q = [&](auto dt_tag) __attribute__((always_inline)) {
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh) {
-        const int64_t base = b * p.q_stride + (int64_t)(first_head(hh) + (live ? col : 0)) * D + 8 * kg;
+        const int lc = live ? col : 0;
+        const int64_t base = col_row(lc) * p.q_stride + (int64_t)col_head(hh, lc) * D + 8 * kg;
 #pragma unroll
         for (int c = 0; c < KSTEPS; ++c) {
           float x[8];
@@ -510,11 +542,12 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       den += sl[row_l][i];
     }
     const float res = num / den;
-    const int head = first_head(hh) + hc;
+    const int head = col_head(hh, hc);
+    const int brow = col_row(hc);
     if (p.direct_out) {
-      store_from_f32(p.out, b * p.out_stride + (int64_t)head * D + d, p.q_dtype, res);
+      store_from_f32(p.out, brow * p.out_stride + (int64_t)head * D + d, p.q_dtype, res);
     } else {
-      const int64_t row = ((int64_t)b * p.num_q_heads + head) * p.max_partitions + part;
+      const int64_t row = ((int64_t)brow * p.num_q_heads + head) * p.max_partitions + part;
       p.ws_out[row * D + d] = res;
       if (d == 0) {
         float mo = sm[row_l][0];

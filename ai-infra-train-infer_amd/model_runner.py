@@ -50,6 +50,9 @@ class ModelRunnerConfig:
     device: str = "cuda"
     enable_cuda_graph: bool = True
     max_cuda_graph_batch_size: int = 64
+    # decode steps look for rows that share prefixes as the same blocks (n samples of a prompt,
+    # forks of a cached prefix) and read a shared partition once per group; eager steps only
+    share_prefix_decode: bool = False
 
 
 def slots_for_range(block_table, start, end, block_size):
@@ -323,11 +326,17 @@ class ModelRunner:
             pos[i] = position
             slots[i] = seq["block_table"][-1] * self.block_size + last - 1
             lens[i] = len(toks)
+        groups = None
+        if getattr(self.config, "share_prefix_decode", False) and self._device() != "cpu":
+            from .attention import prepare_prefix_groups
+            groups = prepare_prefix_groups([seq["block_table"] for seq in sequences], lens.tolist(), self.block_size,
+                                           self.config.num_heads, self.config.num_kv_heads, self._device())
         set_context(
             is_prefill=False,
             slot_mapping=self._to_device(slots, torch.int32),
             context_lens=self._to_device(lens, torch.int32),
             block_tables=self._prepare_block_tables(sequences),
+            prefix_groups=groups,
         )
         return self._to_device(ids, torch.long), self._to_device(pos, torch.long)
 

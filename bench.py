@@ -258,6 +258,15 @@ def other_decode_configs(pa, torch, dev, launches):
     unique_tokens = 32 * 1024 + sum(suf)
     meta["cfg4"] = dict(workload="32 prompts x 8 samples, shared 1024-token prefix, suffix U[64,512] (seed 1004), FP16 KV",
                         kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
+    # the same batch with the samples of a prompt named as a group: partitions inside the shared prefix are
+    # read once per prompt (what ModelRunnerConfig.share_prefix_decode does from the host's block-id lists)
+    groups4 = [(8 * i, 8, 1024) for i in range(32)]
+    desc4 = pa.shared_prefix_descriptors(groups4, 256, dev, 512)
+    fns["cfg4_shared_prefix"] = lambda: pa.paged_decode_shared_prefix(
+        w4["q"], w4["k_cache"], w4["v_cache"], w4["block_tables"], w4["context_lens"], scale, groups4,
+        partition_size=512, out=w4["out"], descriptors=desc4)
+    meta["cfg4_shared_prefix"] = dict(workload=meta["cfg4"]["workload"] + "; shared partitions (512 tokens) read once per prompt, "
+                                      "matrix kernel + merge", kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
     t = time_alternating(torch, fns, launches)
     for name, m in meta.items():

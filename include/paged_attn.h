@@ -195,6 +195,54 @@ int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const
                        void* stream);
 
 /*
+ * Partitioned decode for batches whose rows share prefixes as the same physical blocks (n samples
+ * of one prompt, sequences forked from a cached prefix): partitions that lie wholly inside a
+ * group's shared prefix are computed once for all the group's rows - their K and V leave HBM and
+ * the L2 once per group instead of once per row - and every row's remaining partitions as usual;
+ * the merge is pa_merge's.  Same result as pa_decode with the same partition_size.
+ * Replaces: the same reference code as pa_decode (src/inference/attention.py:434-626); the
+ * reference reads a shared block once per sequence that maps it (kv_cache.py:95-101 shares them).
+ * Arguments as pa_decode (partition_size > 0; the matrix kernel, one KV head per wave), plus:
+ *   group_desc            device int32 [num_groups][4]: first batch row, number of rows (consecutive),
+ *                         shared partitions, unused.  The first shared_partitions x partition_size
+ *                         tokens of every row of a group must map to the same physical blocks as
+ *                         the group's first row, and every row's context must hold them.
+ *   max_group_rows        most rows of any group; rows x (num_q_heads / num_kv_heads) <= 16
+ *   max_shared_partitions most shared partitions of any group
+ *   row_skip              device int32 [batch]: the row's group's shared partitions, 0 for rows of
+ *                         no group
+ *   max_own_partitions    most partitions any row computes itself:
+ *                         >= ceil(context_len / partition_size) - row_skip[row] for every row
+ * The launch trusts the descriptors (pa_check_shared_prefix counts what is wrong with them).
+ */
+int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
+                            const void* v_cache, const float* k_scale, const float* v_scale,
+                            int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
+                            int64_t table_width, const int32_t* context_lens, void* out,
+                            int64_t out_token_stride, int64_t batch, int64_t num_q_heads,
+                            int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                            int64_t num_blocks, float scale, int64_t partition_size,
+                            int64_t max_partitions, void* workspace, int64_t workspace_bytes,
+                            int waves_per_workgroup, const int32_t* group_desc, int64_t num_groups,
+                            int64_t max_group_rows, int64_t max_shared_partitions,
+                            const int32_t* row_skip, int64_t max_own_partitions, void* stream);
+
+/*
+ * Debug aid for pa_decode_shared_prefix: counts, on the device, what is wrong with its descriptors.
+ *   counts[0] += table entries inside a group's shared partitions that differ between a row and
+ *                the group's first row (or lie beyond table_width)
+ *   counts[1] += rows whose context is shorter than their group's shared tokens or whose row_skip
+ *                is not their group's shared partitions; groups that reach outside the batch
+ *   counts[2] += rows of no group with a non-zero row_skip, rows claimed by two groups
+ * counts is a device int32[3] that the caller clears beforehand and reads afterwards.
+ * No counterpart in the reference.
+ */
+int pa_check_shared_prefix(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
+                           const int32_t* context_lens, int64_t batch, int64_t block_size,
+                           int64_t partition_size, const int32_t* group_desc, int64_t num_groups,
+                           const int32_t* row_skip, int32_t* counts, void* stream);
+
+/*
  * Timing aid: the launch of pa_decode_partials with the attention arithmetic taken out.  Every
  * K, V, scale and table load of the real launch is issued from the same lanes in the same order
  * and every loaded word is consumed (a checksum lands in `workspace`), but no dot product,

@@ -94,3 +94,43 @@ def test_graph_runner_host_side_without_a_gpu():
     assert st == {"captured_sizes": [], "total_captures": 0, "total_replays": 0, "graph_pool_active": False,
                   "supported_batch_sizes": [1, 2, 4, 8, 16]}
     r.invalidate()
+
+
+def test_find_prefix_groups(pa):
+    f = pa.find_prefix_groups
+    shared = list(range(100, 140))                       # 40 blocks = 640 tokens
+    rows = [shared + [200 + i] for i in range(8)] + [[300, 301]] + [shared[:20] + [400]]
+    lens = [650] * 8 + [20] + [330]
+    # 8 samples of one prompt, a loner, a row that shares half of the prompt with nobody next to it
+    assert f(rows, lens, 16, 16, 8, 128) == [(0, 8, 640)]
+    # whole partitions only: 640 shared tokens hold two partitions of 256
+    assert f(rows, lens, 16, 16, 8, 256) == [(0, 8, 512)]
+    # four query heads per KV head: at most four rows per group
+    assert f(rows, lens, 16, 32, 8, 128) == [(0, 4, 640), (4, 4, 640)]
+    # more than 8 query heads per KV head: no room for a second row
+    assert f(rows, lens, 16, 128, 8, 128) == []
+    # a row whose context ends inside the shared blocks caps what its group shares
+    assert f(rows[:3], [650, 300, 650], 16, 16, 8, 128) == [(0, 3, 256)]
+    # a run ends where the next row would shrink the shared part by more than it adds
+    two_prompts = [shared + [1]] * 4 + [shared[:8] + list(range(500, 532)) + [2]] * 4
+    assert f(two_prompts, [650] * 8, 16, 16, 8, 128) == [(0, 4, 640), (4, 4, 640)]
+    # nothing shared, or less than a partition
+    assert f([[1, 2, 3], [4, 5, 6]], [48, 48], 16, 16, 8, 32) == []
+    assert f([[1, 2, 3], [1, 5, 6]], [48, 48], 16, 16, 8, 32) == []
+    assert f([], [], 16, 16, 8) == []
+
+
+def test_shared_prefix_descriptors_and_context_field(pa):
+    desc, skip, max_rows, max_parts, min_skip = pa.shared_prefix_descriptors([(0, 3, 512), (5, 2, 1024)], 8, "cpu", 256)
+    assert desc.dtype == torch.int32 and desc.tolist() == [[0, 3, 2, 0], [5, 2, 4, 0]]
+    assert skip.tolist() == [2, 2, 2, 0, 0, 4, 4, 0] and (max_rows, max_parts, min_skip) == (3, 4, 0)
+    assert pa.shared_prefix_descriptors([(0, 2, 512)], 2, "cpu", 256)[4] == 2        # every row skips two
+    with pytest.raises(RuntimeError, match="outside the batch"):
+        pa.shared_prefix_descriptors([(7, 2, 512)], 8, "cpu", 256)
+    assert pa.prepare_prefix_groups([[1, 2], [3, 4]], [32, 32], 16, 16, 8, "cpu", 32) is None
+    pg = pa.prepare_prefix_groups([[1, 2, 9], [1, 2, 8]], [40, 40], 16, 16, 8, "cpu", 32)
+    assert pg["groups"] == [(0, 2, 32)] and pg["partition_size"] == 32
+    pa.set_context(False, context_lens=torch.ones(2, dtype=torch.int32), prefix_groups=pg)
+    assert pa.get_context().prefix_groups is pg
+    pa.reset_context()
+    assert pa.get_context().prefix_groups is None
