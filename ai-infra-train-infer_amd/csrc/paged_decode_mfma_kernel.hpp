@@ -39,7 +39,6 @@ typedef _Float16 mhalf8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 mhalf4_t __attribute__((ext_vector_type(4)));
 typedef __fp16 mfp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef float mfloat4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t muint2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kMfmaTile = 32;    // tokens per tile
 constexpr int kMfmaHeads = 16;   // query-head columns of the matrix operand
