@@ -157,6 +157,13 @@ def test_k_samples_share_prompt_blocks_and_decode_like_private_copies(pa, gpu, c
         want = oracle.decode(q, pk, pv, pbt, ctx, scale, pks, pvs, cache)
         tol = dict(rtol=1e-2, atol=1e-2) if cache == "fp8" else dict(rtol=1e-3, atol=2e-3)
         torch.testing.assert_close(got.float(), want.float(), **tol)
+        # the same step with the samples of a prompt found as groups in the manager's tables: the shared
+        # full blocks of a prompt are read once per prompt
+        groups = pa.find_prefix_groups([mgr.get_block_table(s) for s in seqs], lens, BS, HQ, HKV, 32)
+        assert groups == [(0, SAMPLES, 32), (SAMPLES, SAMPLES, 64), (2 * SAMPLES, SAMPLES, 128)]
+        shared = pa.paged_decode_shared_prefix(q.to(gpu), kc, vc, bt.to(gpu), ctx.to(gpu), scale, groups, ks, vs,
+                                               partition_size=32).cpu()
+        torch.testing.assert_close(shared.float(), want.float(), **tol)
 
     for s in seqs:
         mgr.free_sequence(s)
