@@ -355,6 +355,39 @@ def prefill_cfg5a(pa, torch, dev, steps, warmup, constant_data=False):
             "frac_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4)}
 
 
+def prefill_other_cache_types(pa, torch, dev, steps, warmup):
+    """The chunked-prefill launch of configuration 5a over a bf16 and an fp8 cache (staged through
+    registers and converted to fp16 on the way into LDS) beside the fp16 one (global -> LDS directly),
+    alternated in one timed loop."""
+    S, CACHED, NEW, HQ, HKV, D, BS = 8, 2048, 512, 16, 8, 128, 16
+    g = torch.Generator(device=dev).manual_seed(1005)
+    bps = (CACHED + NEW) // BS
+    nb = S * bps + 32
+    tables = torch.randperm(nb, generator=g, device=dev)[:S * bps].view(S, bps).to(torch.int32).contiguous()
+    q = torch.randn(S * NEW, HQ, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    cu_q = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * NEW
+    cu_k = torch.arange(0, S + 1, device=dev, dtype=torch.int32) * (CACHED + NEW)
+    out = torch.empty_like(q)
+    fns = {}
+    for kind in ("fp16", "bf16", "fp8"):
+        kc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32)
+        vc = torch.randn(nb, BS, HKV, D, generator=g, device=dev, dtype=torch.float32)
+        ks = vs = None
+        if kind == "fp16":
+            kc, vc = kc.half(), vc.half()
+        elif kind == "bf16":
+            kc, vc = kc.bfloat16(), vc.bfloat16()
+        else:
+            kc, vc = kc.to(torch.float8_e4m3fn), vc.to(torch.float8_e4m3fn)
+            ks = torch.rand(nb, BS, device=dev) + 0.5
+            vs = torch.rand(nb, BS, device=dev) + 0.5
+        fns[kind] = lambda kc=kc, vc=vc, ks=ks, vs=vs: pa.paged_prefill(q, kc, vc, cu_q, cu_k, NEW, D ** -0.5,
+                                                                        block_tables=tables, k_scale=ks, v_scale=vs, out=out)
+    t = time_alternating(torch, fns, steps, warmup=max(warmup, 20))
+    return {"workload": "8 x (2048 cached + 512 new), 16q/8kv, d128, bf16 Q; cache element type varied",
+            "us": {k: spread(v) for k, v in t.items()}}
+
+
 def hbm_stream_read(pa, torch, dev, launches):
     """The plain read rate of the GPU: pa_hbm_read_probe over a 1 GiB buffer (every workgroup streams
     its own contiguous share once, 16-byte loads), for four workgroup counts, alternated, medians.
@@ -907,6 +940,7 @@ def main():
             "what": "the prefill launch above with Q, K and V all ones: the same instructions on operands that do "
                     "not toggle; the difference to `prefill_mfma` is clock throttling under the matrix pipe",
             "us": const["us"], "tflops": const["tflops"], "frac_mfma_peak": const["frac_mfma_peak"]}
+        line["prefill_other_cache_types"] = prefill_other_cache_types(pa, torch, dev, launches, max(20, args.warmup))
         line["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup)
         line["kv_gather"] = kv_gather_times(pa, torch, dev, args.steps, args.warmup)
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
