@@ -297,14 +297,20 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
     slices = (g + kMatrixPath - 1) / kMatrixPath;
     // One KV head per wave.  4-wave workgroups (two share a CU) are the best or within 3 % of the best
     // shape from batch 8 x 320 to batch 256 x 1k tokens; launches with fewer workgroups than CUs put
-    // 8 waves on the CUs they do reach.  Two heads per wave gain nothing here: the wave's longer
-    // chain of products per tile costs what the wider pieces save.
+    // 8 waves on the CUs they do reach.  Two heads per wave (256-byte pieces of an fp8 row, 32 KiB of
+    // LDS per wave, so one 4-wave workgroup per CU) pay in one case only: an fp8 cache and a halved
+    // grid that is just one workgroup per CU (batch 64 x 8 KV heads: 103-105 against 112-115 us);
+    // with fewer workgroups they idle CUs, with more the second round costs what the pieces save.
     s.hpw = kv_heads_per_wave == 2 ? 2 : 1;
+    const int64_t cus = compute_units();
+    const int64_t unpaired = num_kv_heads * slices * max_partitions * batch;
+    if (kv_heads_per_wave == 0 && kv == KV_FP8 && num_kv_heads % 2 == 0 && !shared && (waves == 0 || waves == 4) &&
+        unpaired / 2 <= cus && unpaired / 2 * 10 >= cus * 9)
+      s.hpw = 2;
     if (waves != 0) {
       s.waves = waves;
     } else {
-      const int64_t wgs = (num_kv_heads / s.hpw) * slices * max_partitions * batch;
-      s.waves = (s.hpw == 1 && wgs < compute_units() && !shared) ? 8 : 4;
+      s.waves = (s.hpw == 1 && unpaired < cus && !shared) ? 8 : 4;
     }
   } else {
     if (q_heads_per_wave != 0) {
