@@ -201,7 +201,8 @@ int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const
  * the L2 once per group instead of once per row - and every row's remaining partitions as usual;
  * the merge is pa_merge's.  Same result as pa_decode with the same partition_size.
  * Replaces: the same reference code as pa_decode (src/inference/attention.py:434-626); the
- * reference reads a shared block once per sequence that maps it (kv_cache.py:95-101 shares them).
+ * reference reads a shared block once per sequence that maps it (blocks carry a ref_count for
+ * prefix sharing, src/inference/kv_cache.py:42-62, 190-210).
  * Arguments as pa_decode (partition_size > 0; the matrix kernel, one KV head per wave), plus:
  *   group_desc            device int32 [num_groups][4]: first batch row, number of rows (consecutive),
  *                         shared partitions, unused.  The first shared_partitions x partition_size
