@@ -380,6 +380,7 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
   hipStream_t st = (hipStream_t)stream;
   p.inner = (int)(num_kv_heads / s.hpw) * slices;
   p.probe = mode == kDecodeProbe ? 1 : 0;
+  p.batch = (int)batch;
   p.group_desc = nullptr;
   p.row_skip = nullptr;
   p.num_prefix_wgs = p.prefix_parts = p.suffix_parts = 0;

@@ -249,7 +249,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       ids[x] = bt_row[min(tok >> p.bs_log2, last_blk)];
     }
   };
-  auto issue = [&](TileT& t, int tile, const int (&ids)[4]) __attribute__((always_inline)) {
+  auto issue_as = [&](auto stream_tag, TileT& t, int tile, const int (&ids)[4]) __attribute__((always_inline)) {
+    constexpr bool STREAM = decltype(stream_tag)::value;
     if constexpr (LM) {
 #pragma unroll
       for (int sb = 0; sb < NSUB; ++sb) {
@@ -265,8 +266,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
         for (int r = 0; r < 4; ++r) {
 #pragma unroll
           for (int c = 0; c < G::NLD; ++c) {
-            load_words<G::LB>(kp + (r * token_bytes + c * G::LPR * G::LB), &t.k[4 * sb + r][c * (G::LB / 4)]);
-            load_words<G::LB>(vp + (r * token_bytes + c * G::LPR * G::LB), &t.v[4 * sb + r][c * (G::LB / 4)]);
+            load_words<G::LB, STREAM>(kp + (r * token_bytes + c * G::LPR * G::LB), &t.k[4 * sb + r][c * (G::LB / 4)]);
+            load_words<G::LB, STREAM>(vp + (r * token_bytes + c * G::LPR * G::LB), &t.v[4 * sb + r][c * (G::LB / 4)]);
           }
         }
         const uint64_t slot = ((uint64_t)phys << p.bs_log2) + off;
@@ -285,8 +286,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
         const uint8_t* vp = p.v_cache + base;
 #pragma unroll
         for (int c = 0; c < G::NLD; ++c) {
-          load_words<G::LB>(kp + (lane_off + c * G::LPR * G::LB), &t.k[r][c * (G::LB / 4)]);
-          load_words<G::LB>(vp + (lane_off + c * G::LPR * G::LB), &t.v[r][c * (G::LB / 4)]);
+          load_words<G::LB, STREAM>(kp + (lane_off + c * G::LPR * G::LB), &t.k[r][c * (G::LB / 4)]);
+          load_words<G::LB, STREAM>(vp + (lane_off + c * G::LPR * G::LB), &t.v[r][c * (G::LB / 4)]);
         }
       }
     }
@@ -485,26 +486,35 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   // ---- this wave's tiles: wave, wave + W, ... -------------------------------------------------------
   const int n_mine = ntiles > wave ? (ntiles - wave + W - 1) / W : 0;
   const bool has_tail = ((end - begin) % TILE) != 0;
-  if (n_mine > 0) {
-    // The table entries of the tile after next are asked for before the wait for this tile's data:
-    // scalar loads share a counter with the LDS reads, and an outstanding one would hold up the
-    // first product (fp8, two heads per wave: 108 -> 100.5 us at batch 64 x 4096 tokens).
-    TileT t;
-    int ids[4], ids_next[4];
-    load_ids(wave, ids);
-    issue(t, wave, ids);
-    if (n_mine > 1) load_ids(wave + W, ids);
-    for (int i = 0; i < n_mine; ++i) {
-      const int tile = wave + i * W;
-      const bool masked = has_tail && tile == ntiles - 1;
-      if (i + 2 < n_mine) load_ids(tile + 2 * W, ids_next);
-      write_tile(t, tile, masked);
-      if (i + 1 < n_mine) issue(t, tile + W, ids);
-      compute(tile, masked);
+  // The loop exists twice, with streaming and with ordinary loads (see load_words), chosen once per
+  // workgroup: a group's shared partitions are read once for all its rows and stream; a row's own
+  // token range streams unless a neighbouring row maps its first block too.
+  auto run_tiles = [&](auto stream_tag) __attribute__((always_inline)) {
+    if (n_mine > 0) {
+      // The table entries of the tile after next are asked for before the wait for this tile's data:
+      // scalar loads share a counter with the LDS reads, and an outstanding one would hold up the
+      // first product (fp8, two heads per wave: 108 -> 100.5 us at batch 64 x 4096 tokens).
+      TileT t;
+      int ids[4], ids_next[4];
+      load_ids(wave, ids);
+      issue_as(stream_tag, t, wave, ids);
+      if (n_mine > 1) load_ids(wave + W, ids);
+      for (int i = 0; i < n_mine; ++i) {
+        const int tile = wave + i * W;
+        const bool masked = has_tail && tile == ntiles - 1;
+        if (i + 2 < n_mine) load_ids(tile + 2 * W, ids_next);
+        write_tile(t, tile, masked);
+        if (i + 1 < n_mine) issue_as(stream_tag, t, tile + W, ids);
+        compute(tile, masked);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) ids[x] = ids_next[x];
+        for (int x = 0; x < 4; ++x) ids[x] = ids_next[x];
+      }
     }
-  }
+  };
+  if (members > 1 || decode_range_is_private(bt_row, p.bt_stride, b, p.batch, min(begin >> p.bs_log2, last_blk)))
+    run_tiles(std::true_type{});
+  else
+    run_tiles(std::false_type{});
 
   // ---- merge the waves: common reference, then plain sums ---------------------------------------------
 #pragma unroll
