@@ -67,7 +67,7 @@ SIGNATURES = {
     "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_check_tables": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
     "pa_mfma_rate_probe": (_i64, [_ptr, _i64, _ptr, _ptr]),
-    "pa_hbm_read_probe": (_i64, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "pa_hbm_read_probe": (_i64, [_ptr, _i64, _i64, _int, _ptr, _ptr]),
 }
 
 _lock = threading.Lock()

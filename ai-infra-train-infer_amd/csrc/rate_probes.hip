@@ -6,9 +6,9 @@
 // v_mfma_f32_32x32x16_f16 on every SIMD of the GPU (8 waves per CU, four accumulator chains per
 // wave, operands from registers) on operands the caller supplies - constant ones, or the kind of
 // data the attention kernels see - so that a benchmark can put the sustained rate beside the
-// nominal one.  pa_hbm_read_probe streams a buffer once with 16-byte loads, every workgroup its own
-// contiguous chunk, four loads per lane in flight: the plain read rate of the GPU, which the decode
-// kernels' achieved bytes per second are put beside.  No counterparts in the reference.
+// nominal one.  pa_hbm_read_probe streams a buffer once with 16-byte loads (ordinary or non-temporal),
+// every workgroup its own contiguous chunk, four loads per lane in flight: the plain read rate of the
+// GPU, which the decode kernels' achieved bytes per second are put beside.  No counterparts in the reference.
 #include "pa_common.hpp"
 #include "pa_host.hpp"
 
@@ -45,24 +45,25 @@ __global__ __launch_bounds__(512, 1) void mfma_rate_probe_kernel(const _Float16*
   if (threadIdx.x == 0) sink[blockIdx.x] = r;   // keeps the products alive
 }
 
-// Every workgroup reads `per_group` uint4 words starting at its own offset and leaves the XOR of
-// all of them (folded to one word per workgroup) in `sink`.
-__global__ __launch_bounds__(256) void hbm_read_probe_kernel(const uint4* __restrict__ src, int64_t per_group, uint32_t* sink) {
-  const uint4* q = src + (int64_t)blockIdx.x * per_group;
-  uint4 acc = make_uint4(0u, 0u, 0u, 0u);
+// Every workgroup reads `per_group` 16-byte words starting at its own offset and leaves the XOR of
+// all of them (folded to one word per workgroup) in `sink`.  STREAM: non-temporal loads, as the
+// decode kernels read private K/V.
+template <bool STREAM>
+__global__ __launch_bounds__(256) void hbm_read_probe_kernel(const uint8_t* __restrict__ src, int64_t per_group, uint32_t* sink) {
+  typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+  const u4_t* q = (const u4_t*)src + (int64_t)blockIdx.x * per_group;
+  auto ld = [&](int64_t i) __attribute__((always_inline)) -> u4_t {
+    if constexpr (STREAM) return __builtin_nontemporal_load(q + i);
+    else return q[i];
+  };
+  u4_t acc = {0u, 0u, 0u, 0u};
   int64_t i = threadIdx.x;
   for (; i + 3 * 256 < per_group; i += 4 * 256) {
-    const uint4 a = q[i], b = q[i + 256], c = q[i + 512], d = q[i + 768];
-    acc.x ^= a.x ^ b.x ^ c.x ^ d.x;
-    acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
-    acc.z ^= a.z ^ b.z ^ c.z ^ d.z;
-    acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
+    const u4_t a = ld(i), b = ld(i + 256), c = ld(i + 512), d = ld(i + 768);
+    acc ^= a ^ b ^ c ^ d;
   }
-  for (; i < per_group; i += 256) {
-    const uint4 a = q[i];
-    acc.x ^= a.x; acc.y ^= a.y; acc.z ^= a.z; acc.w ^= a.w;
-  }
-  uint32_t x = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  for (; i < per_group; i += 256) acc ^= ld(i);
+  uint32_t x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) x ^= __shfl_xor(x, off);
   __shared__ uint32_t part[4];
@@ -75,14 +76,19 @@ __global__ __launch_bounds__(256) void hbm_read_probe_kernel(const uint4* __rest
 
 using namespace pa;
 
-extern "C" int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, uint32_t* sink, void* stream) {
+extern "C" int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, int streaming, uint32_t* sink,
+                                     void* stream) {
   if (!src || !sink) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: null pointer");
   if (groups <= 0 || groups > 0x7fffffff || bytes <= 0) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: bad size");
   if (!aligned16(src)) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: buffer must be 16-byte aligned");
   const int64_t per_group = bytes / 16 / groups;
   if (per_group <= 0) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: fewer than 16 bytes per workgroup");
-  hipLaunchKernelGGL(hbm_read_probe_kernel, dim3((unsigned)groups), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4*)src, per_group, sink);
+  if (streaming)
+    hipLaunchKernelGGL(hbm_read_probe_kernel<true>, dim3((unsigned)groups), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t*)src, per_group, sink);
+  else
+    hipLaunchKernelGGL(hbm_read_probe_kernel<false>, dim3((unsigned)groups), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t*)src, per_group, sink);
   const int rc = check_launch("pa_hbm_read_probe");
   if (rc != PA_OK) return rc;
   return per_group * groups * 16;   // bytes read

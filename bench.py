@@ -399,21 +399,24 @@ def hbm_stream_read(pa, torch, dev, launches):
     stream = torch.cuda.current_stream(dev).cuda_stream
     cus = pa.attention._compute_units(dev)
     fns = {}
-    for mult in (2, 8, 32, 128):
-        groups = cus * mult
+    for streaming in (1, 0):
+        for mult in (2, 8, 32, 128):
+            groups = cus * mult
 
-        def fn(groups=groups):
-            got = lib.pa_hbm_read_probe(buf.data_ptr(), nbytes, groups, sink.data_ptr(), stream)
-            assert got == nbytes, lib.pa_last_error()
+            def fn(groups=groups, streaming=streaming):
+                got = lib.pa_hbm_read_probe(buf.data_ptr(), nbytes, groups, streaming, sink.data_ptr(), stream)
+                assert got == nbytes, lib.pa_last_error()
 
-        fns["workgroups_%d" % groups] = fn
+            fns["%sworkgroups_%d" % ("" if streaming else "ordinary_loads_", groups)] = fn
     t = time_alternating(torch, fns, max(20, launches // 5), warmup=3)
-    out = {"what": "pa_hbm_read_probe: 1 GiB streamed once per launch, contiguous share per workgroup, 16-byte loads",
-           "bytes": nbytes}
+    out = {"what": "pa_hbm_read_probe: 1 GiB streamed once per launch, contiguous share per workgroup, 16-byte "
+                   "non-temporal loads (the way the decode kernels read private K/V); ordinary_loads_*: the same "
+                   "with ordinary loads", "bytes": nbytes}
     for name, v in t.items():
         out[name] = {"us": spread(v), "gbps": round(nbytes / med(v) / 1e3, 1),
                      "frac_of_8TBps": round(nbytes / med(v) / 1e3 / HBM_PEAK_GBPS, 4)}
     out["best_gbps"] = max(v["gbps"] for k, v in out.items() if k.startswith("workgroups_"))
+    out["best_gbps_ordinary_loads"] = max(v["gbps"] for k, v in out.items() if k.startswith("ordinary_loads_"))
     del buf
     torch.cuda.empty_cache()
     return out

@@ -275,11 +275,13 @@ int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t steps, float* sink,
 
 /*
  * Measuring aid: the plain read rate of the GPU.  `groups` workgroups of 256 threads each stream
- * their own contiguous share of `bytes` bytes at `src` once (16-byte loads, four per lane in flight)
+ * their own contiguous share of `bytes` bytes at `src` once (16-byte loads, four per lane in flight;
+ * streaming != 0: non-temporal loads, the way the decode kernels read private K and V)
  * and leave the XOR of their words, folded to 32 bits, in sink[group].  Returns the number of bytes
  * read (bytes rounded down to 16 x groups), or a negative error code.  No counterpart in the reference.
  */
-int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, uint32_t* sink, void* stream);
+int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, int streaming, uint32_t* sink,
+                          void* stream);
 
 /*
  * Merge reduction over partitions.

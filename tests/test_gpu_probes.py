@@ -32,9 +32,9 @@ def test_hbm_read_probe_reads_every_word_once(pa, lib, gpu):
     words = torch.randint(-2 ** 31, 2 ** 31 - 1, (1 << 18,), generator=g, dtype=torch.int64).to(torch.int32)
     buf = words.to(gpu)
     stream = torch.cuda.current_stream(gpu).cuda_stream
-    for groups in (1, 7, 64, 1000):
+    for groups, streaming in ((1, 0), (7, 1), (64, 0), (64, 1), (1000, 1)):
         sink = torch.zeros(groups, dtype=torch.int32, device=gpu)
-        got = lib.pa_hbm_read_probe(buf.data_ptr(), buf.numel() * 4, groups, sink.data_ptr(), stream)
+        got = lib.pa_hbm_read_probe(buf.data_ptr(), buf.numel() * 4, groups, streaming, sink.data_ptr(), stream)
         torch.cuda.synchronize()
         per = (buf.numel() // 4 // groups) * 4              # int32 words per workgroup
         assert got == per * groups * 4
@@ -43,8 +43,8 @@ def test_hbm_read_probe_reads_every_word_once(pa, lib, gpu):
         for j in range(1, per):                              # XOR fold on the host
             acc ^= want[:, j]
         assert torch.equal(sink.cpu(), acc), groups
-    assert lib.pa_hbm_read_probe(buf.data_ptr(), 8, 1, sink.data_ptr(), stream) == -1
-    assert lib.pa_hbm_read_probe(None, 1024, 1, sink.data_ptr(), stream) == -1
+    assert lib.pa_hbm_read_probe(buf.data_ptr(), 8, 1, 1, sink.data_ptr(), stream) == -1
+    assert lib.pa_hbm_read_probe(None, 1024, 1, 0, sink.data_ptr(), stream) == -1
 
 
 def test_decode_load_probe_runs_the_decode_launch_shape(pa, lib, gpu):
