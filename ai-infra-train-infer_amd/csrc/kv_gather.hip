@@ -46,10 +46,17 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(const uint8_t* __restric
       const int blk = col < table_width ? block_tables[(int64_t)b * bt_stride + col] : -1;
       if (blk >= 0 && blk < num_blocks) {
         const int64_t slot = (int64_t)blk * block_size + pos % block_size;
-        v = *(const uint4*)(cache + slot * token_bytes + (int64_t)h * row_bytes + (c << 4));
+        // read once per launch: a streaming (non-temporal) load
+        typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+        const u4_t w = __builtin_nontemporal_load((const u4_t*)(cache + slot * token_bytes + (int64_t)h * row_bytes + (c << 4)));
+        v = make_uint4(w[0], w[1], w[2], w[3]);
       }
     }
-    *(uint4*)(out + (((int64_t)b * num_kv_heads + h) * out_len + pos) * row_bytes + (c << 4)) = v;
+    {
+      typedef uint32_t u4s_t __attribute__((ext_vector_type(4)));
+      const u4s_t w2 = {v.x, v.y, v.z, v.w};
+      __builtin_nontemporal_store(w2, (u4s_t*)(out + (((int64_t)b * num_kv_heads + h) * out_len + pos) * row_bytes + (c << 4)));
+    }
   }
 }
 
