@@ -260,13 +260,15 @@ def other_decode_configs(pa, torch, dev, launches):
                         kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
     # the same batch with the samples of a prompt named as a group: partitions inside the shared prefix are
     # read once per prompt (what ModelRunnerConfig.share_prefix_decode does from the host's block-id lists)
-    groups4 = [(8 * i, 8, 1024) for i in range(32)]
-    desc4 = pa.shared_prefix_descriptors(groups4, 256, dev, 512)
+    host_tables = [row[:(n + BS - 1) // BS] for row, n in zip(w4["block_tables"].cpu().tolist(), lens4)]
+    pg4 = pa.prepare_prefix_groups(host_tables, lens4, BS, HQ, HKV, dev)
+    assert pg4 is not None and pg4["groups"] == [(8 * i, 8, 1024) for i in range(32)], pg4 and pg4["groups"]
     fns["cfg4_shared_prefix"] = lambda: pa.paged_decode_shared_prefix(
-        w4["q"], w4["k_cache"], w4["v_cache"], w4["block_tables"], w4["context_lens"], scale, groups4,
-        partition_size=512, out=w4["out"], descriptors=desc4)
-    meta["cfg4_shared_prefix"] = dict(workload=meta["cfg4"]["workload"] + "; shared partitions (512 tokens) read once per prompt, "
-                                      "matrix kernel + merge", kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
+        w4["q"], w4["k_cache"], w4["v_cache"], w4["block_tables"], w4["context_lens"], scale, pg4["groups"],
+        partition_size=pg4["partition_size"], out=w4["out"], descriptors=pg4["descriptors"])
+    meta["cfg4_shared_prefix"] = dict(workload=meta["cfg4"]["workload"] + "; shared partitions (%d tokens, the group finder's "
+                                      "choice) read once per prompt, matrix kernel + merge" % pg4["partition_size"],
+                                      kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
     t = time_alternating(torch, fns, launches)
     for name, m in meta.items():

@@ -128,6 +128,13 @@ def test_shared_prefix_descriptors_and_context_field(pa):
     with pytest.raises(RuntimeError, match="outside the batch"):
         pa.shared_prefix_descriptors([(7, 2, 512)], 8, "cpu", 256)
     assert pa.prepare_prefix_groups([[1, 2], [3, 4]], [32, 32], 16, 16, 8, "cpu", 32) is None
+    # no partition size given: the coarsest of 2048 / 1024 / 512 / 256 that keeps 90 % of the savings
+    shared = list(range(100, 164))                       # 64 blocks = 1024 tokens
+    auto = pa.prepare_prefix_groups([shared[:40] + [7], shared[:40] + [8]], [650, 650], 16, 16, 8, "cpu")
+    assert auto["partition_size"] == 512 and auto["groups"] == [(0, 2, 512)]
+    auto = pa.prepare_prefix_groups([shared + [7], shared + [8]], [1030, 1030], 16, 16, 8, "cpu")
+    assert auto["partition_size"] == 1024 and auto["groups"] == [(0, 2, 1024)]
+    assert pa.prepare_prefix_groups([shared[:10] + [7], shared[:10] + [8]], [170, 170], 16, 16, 8, "cpu") is None
     pg = pa.prepare_prefix_groups([[1, 2, 9], [1, 2, 8]], [40, 40], 16, 16, 8, "cpu", 32)
     assert pg["groups"] == [(0, 2, 32)] and pg["partition_size"] == 32
     pa.set_context(False, context_lens=torch.ones(2, dtype=torch.int32), prefix_groups=pg)
