@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 H, HKV, D, BS = 16, 8, 128, 16
 
 
-def _args(d, c, out):
+def _args(d, c, out, H=H):
     t = d["block_tables"]
     fp8 = c["cache_dtype"] == "fp8"
     return [d["q"].data_ptr(), 0, H * D, d["k_cache"].data_ptr(), d["v_cache"].data_ptr(),
@@ -21,7 +21,7 @@ def _args(d, c, out):
             out.data_ptr(), H * D, t.shape[0], H, HKV, D, BS, c["num_blocks"], c["scale"]]
 
 
-def _both(lib, gpu, c, psize):
+def _both(lib, gpu, c, psize, H=H):
     d = cases.to_device(c, gpu)
     batch = d["q"].shape[0]
     parts = max(1, (d["block_tables"].shape[1] * BS + psize - 1) // psize)
@@ -30,9 +30,9 @@ def _both(lib, gpu, c, psize):
     want = torch.full((batch, H, D), float("nan"), dtype=torch.float16, device=gpu)
     got = torch.full_like(want, float("nan"))
     stream = torch.cuda.current_stream(gpu).cuda_stream
-    rc = lib.pa_decode(*_args(d, c, want), psize, parts, ws.data_ptr(), nbytes, 0, 0, 0, stream)
+    rc = lib.pa_decode(*_args(d, c, want, H), psize, parts, ws.data_ptr(), nbytes, 0, 0, 0, stream)
     assert rc == 0, lib.pa_last_error()
-    rc = lib.pa_decode_noalloc(*_args(d, c, got), psize, parts, 0, 0, 0, stream)
+    rc = lib.pa_decode_noalloc(*_args(d, c, got, H), psize, parts, 0, 0, 0, stream)
     assert rc == 0, lib.pa_last_error()
     torch.cuda.synchronize()
     return got.cpu(), want.cpu()
@@ -49,6 +49,15 @@ def test_two_calls_in_a_row_second_one_smaller(lib, gpu, cache):
         assert not torch.isnan(got).any()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.cuda.memory_allocated(gpu) == allocated_before
+
+
+def test_wide_query_groups_take_the_matrix_kernel_through_the_same_entry_point(lib, gpu):
+    """32 query heads over 8 KV heads: the launch picks the matrix kernel; its partials go to the same array."""
+    for seed, lens, psize in ((904, [2000, 333, 1500], 256), (905, [600], 128)):
+        c = cases.make_case(seed, lens, sum((n + 15) // 16 for n in lens) + 8, num_heads=32)
+        got, want = _both(lib, gpu, c, psize, H=32)
+        assert not torch.isnan(got).any()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
 def test_single_pass_needs_no_scratch_and_oversized_launches_are_refused(lib, gpu):
