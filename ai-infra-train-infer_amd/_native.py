@@ -39,17 +39,14 @@ SIGNATURES = {
                          _int, _int, _int, _ptr]),
     "pa_decode_shared_prefix": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr, _ptr,
                                        _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
-                                       _int, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
-    "pa_check_shared_prefix": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
+                                       _int, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr]),
+    "pa_check_shared_prefix": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
     "pa_decode_noalloc": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
                                  _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64,
                                  _int, _int, _int, _ptr]),
     "pa_decode_partials": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _i64, _ptr, _i64,
                                   _int, _int, _int, _ptr]),
-    "pa_decode_load_probe": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _i64, _ptr,
-                                    _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr, _i64,
-                                    _int, _int, _int, _ptr]),
     "pa_merge": (_int, [_ptr, _i64, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_prefill": (_int, [_ptr, _int, _i64, _ptr, _ptr, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr,
                           _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]),
@@ -66,8 +63,6 @@ SIGNATURES = {
     "pa_decode_advance": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_check_tables": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
-    "pa_mfma_rate_probe": (_i64, [_ptr, _i64, _ptr, _ptr]),
-    "pa_hbm_read_probe": (_i64, [_ptr, _i64, _i64, _int, _ptr, _ptr]),
 }
 
 _lock = threading.Lock()

@@ -6,6 +6,7 @@ runner that binds caches by isinstance() and sets the global context can use the
 unchanged.  Everything computes on the GPU through libpaged_attn.so; a CPU tensor or a
 missing library raises RuntimeError (there is no fallback path).
 """
+import contextlib
 import functools
 import os
 from typing import Optional
@@ -394,25 +395,50 @@ def _device_index(device):
     return device.index if device.index is not None else torch.cuda.current_device()
 
 
-def reserve_decode_workspace(device, nbytes):
-    """Make the device's partition workspace at least `nbytes` large and return it.
+_GRAPHS = "graphs"
+_sizing_for_graphs = 0
 
-    One workspace per device serves every partitioned decode launch on it.  It only grows, and
-    a tensor it has outgrown is kept alive, never handed back to the allocator: a HIP graph
-    recorded earlier still holds that tensor's address.  Growing allocates, so it must happen
-    outside a graph capture - whoever captures decode graphs reserves the largest size first
-    (ModelRunner does, from its largest batch and the launch policy's partition limit); inside a
-    capture a workspace that is too small raises instead of allocating from the graph's pool.
-    Launches that run at the same time on different streams of one device must not share it: give
-    those their own tensor through paged_decode(workspace=...)."""
+
+@contextlib.contextmanager
+def sizing_graph_workspace():
+    """While active, every partitioned decode launch also sizes the workspace that recorded graphs
+    use: wrap the warm-up runs that precede a capture in it."""
+    global _sizing_for_graphs
+    _sizing_for_graphs += 1
+    try:
+        yield
+    finally:
+        _sizing_for_graphs -= 1
+
+
+def reserve_decode_workspace(device, nbytes, for_graphs=False):
+    """Make a partition workspace at least `nbytes` large and return it.
+
+    Workspaces are kept per (device, stream): launches that run at the same time on different
+    streams of one GPU never share partials.  Launches recorded into a HIP graph use one more
+    workspace per device, the graphs' own (for_graphs=True, and whenever the current stream is
+    capturing): a capture runs on a side stream of its own, and the replays may run on any.  Graphs
+    of one device share it, so two graphs replayed at the same time on different streams would
+    race; give such launches their own tensor through paged_decode(workspace=...).
+    A workspace only grows, and a tensor it has outgrown is kept alive, never handed back to the
+    allocator: a recorded graph still holds that tensor's address.  Growing allocates, so it must
+    happen outside a capture - whoever captures decode graphs reserves the largest size first
+    (ModelRunner does, from its largest batch and the launch policy's partition limit; warm-up runs
+    inside sizing_graph_workspace() do it too); inside a capture a workspace that is too small
+    raises instead of allocating from the graph's pool."""
     idx = _device_index(device)
-    held = _WORKSPACES.setdefault(idx, [])
+    capturing = torch.cuda.is_current_stream_capturing()
+    if _sizing_for_graphs and not capturing and not for_graphs:
+        reserve_decode_workspace(device, nbytes, for_graphs=True)
+    key = (idx, _GRAPHS if (for_graphs or capturing) else torch.cuda.current_stream(idx).cuda_stream)
+    held = _WORKSPACES.setdefault(key, [])
     if held and held[-1].numel() >= nbytes:
         return held[-1]
-    if torch.cuda.is_current_stream_capturing():
+    if capturing:
         raise RuntimeError(
-            "paged_decode: the partition workspace of cuda:%d holds %d bytes and this launch needs %d; "
-            "it cannot grow during a graph capture - call reserve_decode_workspace() before capturing"
+            "paged_decode: the graphs' partition workspace of cuda:%d holds %d bytes and this launch needs %d; "
+            "it cannot grow during a graph capture - call reserve_decode_workspace(..., for_graphs=True) or run "
+            "the warm-up inside sizing_graph_workspace() before capturing"
             % (idx, held[-1].numel() if held else 0, nbytes))
     ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=torch.device("cuda", idx))
     held.append(ws)
@@ -567,7 +593,7 @@ def find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_
     of the matrix kernel's operand); longer runs are cut into several groups, and a run ends where
     the next row would shrink what the group shares by more than it adds."""
     max_rows = 16 // max(1, num_q_heads // num_kv_heads)
-    if max_rows < 2:
+    if max_rows < 2 or partition_size <= 0 or partition_size % block_size:
         return []
     part_blocks = partition_size // block_size
     groups, n, b = [], len(block_tables), 0
@@ -594,63 +620,191 @@ def find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_
     return groups
 
 
+def _common_blocks(a, b, cap):
+    """Leading entries, at most cap, that two block-id lists have in common (bisection over slice
+    comparisons, which run at C speed)."""
+    if a[:cap] == b[:cap]:
+        return cap
+    lo, hi = 0, cap                    # a[:lo] == b[:lo], a[:hi] != b[:hi]
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        if a[:mid] == b[:mid]:
+            lo = mid
+        else:
+            hi = mid
+    return lo
+
+
+def find_prefix_groups_anywhere(block_tables, context_lens, block_size, num_q_heads, num_kv_heads,
+                                partition_size=SHARED_PREFIX_PARTITION, rows=None):
+    """find_prefix_groups for rows that share prefixes wherever they sit in the batch, as
+    [([row, ...], shared_tokens)].  Rows that share anything share their first physical block, so
+    the rows are bucketed by it (one dictionary pass; a batch without sharing costs nothing more).
+    A bucket's rows are ordered by their block ids, which puts the longest common prefixes next to
+    each other: what a run of the ordered rows shares is the smallest common prefix of its
+    neighbours, and the cut of the order into runs of at most 16 // (num_q_heads // num_kv_heads)
+    rows that saves the most reads ((rows - 1) x shared partitions per run) is found by dynamic
+    programming.  rows: the batch rows the entries of block_tables belong to (default 0, 1, ...)."""
+    max_rows = 16 // max(1, num_q_heads // num_kv_heads)
+    if max_rows < 2 or partition_size <= 0 or partition_size % block_size:
+        return []
+    part_blocks = partition_size // block_size
+    rows = list(range(len(block_tables))) if rows is None else list(rows)
+    buckets = {}
+    for i, table in enumerate(block_tables):
+        if len(table) and int(context_lens[i]) >= partition_size:
+            buckets.setdefault(table[0], []).append(i)
+    out = []
+    for members in buckets.values():
+        n = len(members)
+        if n < 2:
+            continue
+        members.sort(key=lambda i: block_tables[i])
+        cap = [min(len(block_tables[i]), int(context_lens[i]) // block_size) for i in members]
+        near = [_common_blocks(block_tables[members[k]], block_tables[members[k + 1]], min(cap[k], cap[k + 1]))
+                for k in range(n - 1)]
+        best = [0] * (n + 1)             # best[i]: most partition reads saved by cutting the first i rows
+        cut = [None] * (n + 1)           # the last run of that cut as (start, shared blocks), None: row i - 1 alone
+        for i in range(1, n + 1):
+            best[i], cut[i] = best[i - 1], None
+            shared = cap[i - 1]
+            for j in range(i - 2, max(i - max_rows, 0) - 1, -1):      # the run members[j:i]
+                shared = min(shared, near[j], cap[j])
+                parts = shared // part_blocks
+                if parts < 1:
+                    break
+                gain = best[j] + (i - j - 1) * parts
+                if gain > best[i]:
+                    best[i], cut[i] = gain, (j, shared)
+        i = n
+        while i > 0:
+            if cut[i] is None:
+                i -= 1
+                continue
+            j, shared = cut[i]
+            out.append((sorted(rows[m] for m in members[j:i]), (shared // part_blocks) * partition_size))
+            i = j
+    out.sort(key=lambda g: g[0][0])
+    return out
+
+
+class PrefixGroups:
+    """Device descriptors of a pa_decode_shared_prefix launch.
+
+    group_desc int32 [capacity, 4] (first, rows, shared partitions, 0; groups past num_groups - and
+    any group of 0 partitions - are empty), group_rows int32 [..] or None (None: a group's rows are
+    consecutive batch rows from `first`; else they are group_rows[first : first + rows]), row_skip
+    int32 [batch] (the leading partitions of a row that its group computes).  num_groups,
+    max_group_rows, max_shared_partitions and min_row_skip are the host-side bounds the launch is
+    sized with; a recorded graph fixes them at the descriptors' capacity."""
+
+    def __init__(self, partition_size, group_desc, group_rows, row_skip, num_groups, max_group_rows,
+                 max_shared_partitions, min_row_skip=0, groups=None):
+        self.partition_size = int(partition_size)
+        self.group_desc, self.group_rows, self.row_skip = group_desc, group_rows, row_skip
+        self.num_groups, self.max_group_rows = int(num_groups), int(max_group_rows)
+        self.max_shared_partitions, self.min_row_skip = int(max_shared_partitions), int(min_row_skip)
+        self.groups = groups                   # host copy, for tests and debugging
+
+    @property
+    def batch(self):
+        return self.row_skip.numel()
+
+
+def _normalise_groups(groups):
+    """[(first, rows, tokens)] or [([rows], tokens)] -> ([([rows], tokens)], all consecutive?)"""
+    norm, consecutive = [], True
+    for g in groups:
+        if len(g) == 3:
+            first, count, tokens = g
+            norm.append((list(range(int(first), int(first) + int(count))), int(tokens)))
+        else:
+            members, tokens = g
+            members = [int(r) for r in members]
+            consecutive = consecutive and members == list(range(members[0], members[0] + len(members)))
+            norm.append((members, int(tokens)))
+    return norm, consecutive
+
+
 def shared_prefix_descriptors(groups, batch, device, partition_size=SHARED_PREFIX_PARTITION):
-    """Device descriptors of a pa_decode_shared_prefix launch from [(first_row, rows, shared_tokens)]:
-    (group_desc int32 [G, 4], row_skip int32 [batch], most rows per group, most shared partitions,
-    fewest partitions any row skips)."""
-    desc = torch.zeros((max(len(groups), 1), 4), dtype=torch.int32)
-    skip = torch.zeros(batch, dtype=torch.int32)
-    max_rows = max_parts = 0
-    for i, (first, rows, shared_tokens) in enumerate(groups):
-        parts = int(shared_tokens) // partition_size
-        if first < 0 or rows < 1 or first + rows > batch:
-            raise RuntimeError("shared_prefix_descriptors: group (%d, %d) reaches outside the batch of %d" % (first, rows, batch))
-        desc[i, 0], desc[i, 1], desc[i, 2] = first, rows, parts
-        skip[first:first + rows] = parts
-        max_rows, max_parts = max(max_rows, rows), max(max_parts, parts)
+    """PrefixGroups for [(first_row, rows, shared_tokens)] (find_prefix_groups) or
+    [([row, ...], shared_tokens)] (find_prefix_groups_anywhere): one pinned host buffer, one copy."""
+    norm, consecutive = _normalise_groups(groups)
+    ng = len(norm)
+    host = torch.zeros(4 * max(ng, 1) + 2 * batch, dtype=torch.int32)
+    desc = host[:4 * max(ng, 1)].view(-1, 4)
+    rows_flat = host[4 * max(ng, 1):4 * max(ng, 1) + batch]
+    skip = host[4 * max(ng, 1) + batch:]
+    max_rows = max_parts = cursor = 0
+    for i, (members, shared_tokens) in enumerate(norm):
+        parts = shared_tokens // partition_size
+        if not members or min(members) < 0 or max(members) >= batch:
+            raise RuntimeError("shared_prefix_descriptors: group %s reaches outside the batch of %d" % (members, batch))
+        if cursor + len(members) > batch:
+            raise RuntimeError("shared_prefix_descriptors: rows claimed by more than one group")
+        desc[i, 0] = members[0] if consecutive else cursor
+        desc[i, 1], desc[i, 2] = len(members), parts
+        rows_flat[cursor:cursor + len(members)] = torch.tensor(members, dtype=torch.int32)
+        cursor += len(members)
+        skip[torch.tensor(members, dtype=torch.long)] = parts
+        max_rows, max_parts = max(max_rows, len(members)), max(max_parts, parts)
     min_skip = int(skip.min()) if batch else 0
-    return desc.to(device), skip.to(device), max_rows, max_parts, min_skip
+    dev = host.pin_memory().to(device, non_blocking=True) if torch.device(device).type == "cuda" else host
+    n4 = 4 * max(ng, 1)
+    return PrefixGroups(partition_size, dev[:n4].view(-1, 4), None if consecutive else dev[n4:n4 + batch],
+                        dev[n4 + batch:], ng, max(1, max_rows), max_parts, min_skip, groups=norm)
+
+
+def choose_prefix_partition(find, sizes=(2048, 1024, 512, 256), keep=0.9):
+    """The coarsest partition size of `sizes` whose groups still keep `keep` of the reads that the
+    finest size saves (coarser partitions mean fewer, longer-lived workgroups and fewer partials to
+    merge: the fourth benchmark configuration takes 119 us at 256 tokens, 93 at 512, 87 at 1024).
+    find(size) -> groups as the finders return them.  Returns (size, groups) or (None, [])."""
+    def saved(groups):
+        return sum((len(g[0]) - 1 if len(g) == 2 else g[1] - 1) * g[-1] for g in groups)
+    sizes = sorted(sizes, reverse=True)
+    fine = find(sizes[-1])
+    if not fine:
+        return None, []
+    for size in sizes[:-1]:
+        coarse = find(size)
+        if coarse and saved(coarse) >= keep * saved(fine):
+            return size, coarse
+    return sizes[-1], fine
 
 
 def prepare_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, device,
-                          partition_size=None):
+                          partition_size=None, anywhere=False):
     """What a decode step hands the attention layers (InferenceContext.prefix_groups) when rows share
-    prefixes: the groups found on the host in the per-row block-id lists and their device descriptors,
-    built once per step for all layers.  None when no two rows share a whole partition.
-    partition_size None: the coarsest of 2048, 1024, 512, 256 tokens that still keeps 90 % of the
-    reads that 256-token partitions would save (coarser partitions mean fewer, longer-lived
-    workgroups and fewer partials to merge: config 4 takes 119 us at 256, 93 at 512, 87 at 1024)."""
+    prefixes: the groups found on the host in the per-row block-id lists and their device descriptors
+    (a PrefixGroups), built once per step for all layers.  None when no two rows share a whole
+    partition.  partition_size None: choose_prefix_partition's pick.  anywhere: group rows wherever
+    they sit in the batch (find_prefix_groups_anywhere) instead of runs of consecutive rows."""
+    finder = find_prefix_groups_anywhere if anywhere else find_prefix_groups
+
+    def find(size):
+        if size % block_size:
+            return []
+        return finder(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, size)
+
     if partition_size is None:
-        def saved(groups):
-            return sum((rows - 1) * tokens for _, rows, tokens in groups)
-        fine = find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads,
-                                  SHARED_PREFIX_PARTITION)
-        if not fine:
-            return None
-        groups, partition_size = fine, SHARED_PREFIX_PARTITION
-        for size in (2048, 1024, 512):
-            if size % block_size:
-                continue
-            coarse = find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, size)
-            if coarse and saved(coarse) >= 0.9 * saved(fine):
-                groups, partition_size = coarse, size
-                break
+        partition_size, groups = choose_prefix_partition(find)
     else:
-        groups = find_prefix_groups(block_tables, context_lens, block_size, num_q_heads, num_kv_heads, partition_size)
+        groups = find(int(partition_size))
     if not groups:
         return None
-    return {"groups": groups, "partition_size": int(partition_size),
-            "descriptors": shared_prefix_descriptors(groups, len(block_tables), device, partition_size)}
+    return shared_prefix_descriptors(groups, len(block_tables), device, partition_size)
 
 
 def paged_decode_shared_prefix(q, k_cache, v_cache, block_tables, context_lens, scale, groups, k_scale=None,
                                v_scale=None, partition_size=SHARED_PREFIX_PARTITION, out=None, waves=0,
                                workspace=None, descriptors=None):
     """paged_decode for a batch with shared prefixes: `groups` = [(first_row, rows, shared_tokens)]
-    (find_prefix_groups), or `descriptors` = what shared_prefix_descriptors returned for them (to
-    keep the host-to-device copies out of a step).  Partitions inside a group's shared prefix are
-    read once per group.  Same result as paged_decode(partition_size=partition_size).  The groups
-    are trusted; PA_DEBUG_TABLES=1 checks them against the tables before every launch."""
+    or [([row, ...], shared_tokens)] (the finders above), or `descriptors` = the PrefixGroups made
+    from them (to keep the host-to-device copy out of a step; its partition size then counts).
+    Partitions inside a group's shared prefix are read once per group.  Same result as
+    paged_decode(partition_size=partition_size).  The groups are trusted; PA_DEBUG_TABLES=1 checks
+    them against the tables before every launch."""
     _require_gpu(q, "paged_decode_shared_prefix")
     _require_gpu(k_cache, "paged_decode_shared_prefix")
     _check_cache(k_cache, v_cache, "paged_decode_shared_prefix")
@@ -663,9 +817,14 @@ def paged_decode_shared_prefix(q, k_cache, v_cache, block_tables, context_lens, 
         raise RuntimeError("paged_decode_shared_prefix: q head_dim %d != cache head_dim %d" % (head_dim, d2))
     if block_tables.dim() != 2 or block_tables.shape[0] != batch or context_lens.numel() != batch:
         raise RuntimeError("paged_decode_shared_prefix: block_tables/context_lens do not match the batch")
-    psize = int(partition_size)
+    if descriptors is None:
+        descriptors = shared_prefix_descriptors(groups, batch, q.device, int(partition_size))
+    pg = descriptors
+    psize = pg.partition_size
     if psize <= 0 or psize % 16 or psize % block_size:
         raise RuntimeError("paged_decode_shared_prefix: partition_size must be a multiple of 16 and of the block size")
+    if pg.batch < batch:
+        raise RuntimeError("paged_decode_shared_prefix: descriptors cover %d rows, the batch has %d" % (pg.batch, batch))
     q, qs = _rows(q, "paged_decode_shared_prefix")
     tables = block_tables if block_tables.dtype == torch.int32 else block_tables.to(torch.int32)
     if tables.stride(1) != 1:
@@ -679,18 +838,14 @@ def paged_decode_shared_prefix(q, k_cache, v_cache, block_tables, context_lens, 
     fp8 = kv_code == _native.DTYPE_FP8_E4M3
     if fp8 and (k_scale is None or v_scale is None):
         raise RuntimeError("paged_decode_shared_prefix: fp8 cache needs k_scale and v_scale")
-    if descriptors is None:
-        descriptors = shared_prefix_descriptors(groups, batch, q.device, psize)
-        num_groups = len(groups)
-    else:
-        num_groups = len(groups) if groups is not None else descriptors[0].shape[0]
-    desc, skip, max_rows, max_shared, min_skip = descriptors
     parts = max(1, (tables.shape[1] * block_size + psize - 1) // psize)
+    rows_ptr = pg.group_rows.data_ptr() if pg.group_rows is not None else None
+    rows_len = pg.group_rows.numel() if pg.group_rows is not None else 0
     if _debug_tables():
         counts = torch.zeros(3, dtype=torch.int32, device=q.device)
         rc = lib.pa_check_shared_prefix(tables.data_ptr(), tables.stride(0), tables.shape[1], lens.data_ptr(), batch,
-                                        block_size, psize, desc.data_ptr(), num_groups, skip.data_ptr(),
-                                        counts.data_ptr(), _stream_ptr(q.device))
+                                        block_size, psize, pg.group_desc.data_ptr(), pg.num_groups, rows_ptr, rows_len,
+                                        pg.row_skip.data_ptr(), counts.data_ptr(), _stream_ptr(q.device))
         _native.check(rc, "pa_check_shared_prefix")
         differ, short, stray = counts.tolist()
         if differ or short or stray:
@@ -704,14 +859,16 @@ def paged_decode_shared_prefix(q, k_cache, v_cache, block_tables, context_lens, 
         ws = workspace
     else:
         ws = reserve_decode_workspace(q.device, ws_bytes)
-    own = max(1, parts - min_skip)      # every row computes what its group does not
+    own = max(1, parts - pg.min_row_skip)      # every row computes what its group does not
     rc = lib.pa_decode_shared_prefix(q.data_ptr(), _code(q.dtype, "paged_decode_shared_prefix"), qs, k_cache.data_ptr(),
                                      v_cache.data_ptr(), k_scale.data_ptr() if fp8 else None,
                                      v_scale.data_ptr() if fp8 else None, kv_code, tables.data_ptr(),
                                      tables.stride(0), tables.shape[1], lens.data_ptr(), out.data_ptr(), out.stride(0),
                                      batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, float(scale),
-                                     psize, parts, ws.data_ptr(), ws_bytes, int(waves or 0), desc.data_ptr(), num_groups,
-                                     max(1, max_rows), max_shared, skip.data_ptr(), own, _stream_ptr(q.device))
+                                     psize, parts, ws.data_ptr(), ws_bytes, int(waves or 0), pg.group_desc.data_ptr(),
+                                     pg.num_groups, rows_ptr, rows_len, max(1, pg.max_group_rows),
+                                     min(pg.max_shared_partitions, parts), pg.row_skip.data_ptr(), own,
+                                     _stream_ptr(q.device))
     _native.check(rc, "pa_decode_shared_prefix")
     return out
 
@@ -931,11 +1088,10 @@ class PagedAttention(nn.Module):
         """Rows that share prefixes (ctx.prefix_groups, set by the runner when it found any): the shared
         partitions are read once per group.  None when the step has no groups."""
         pg = getattr(ctx, "prefix_groups", None)
-        if not pg or q.shape[0] != pg["descriptors"][1].numel():
+        if pg is None or q.shape[0] > pg.batch or 16 // max(1, self.num_heads // self.num_kv_heads) < pg.max_group_rows:
             return None
         return paged_decode_shared_prefix(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
-                                          self.scale, pg["groups"], k_scale=ks, v_scale=vs,
-                                          partition_size=pg["partition_size"], descriptors=pg["descriptors"])
+                                          self.scale, None, k_scale=ks, v_scale=vs, descriptors=pg)
 
 
 class PartitionedPagedAttention(PagedAttention):

@@ -1,10 +1,13 @@
-"""Builds libpaged_attn.so (the C-ABI HIP library) for gfx950 with hipcc.
+"""Builds libpaged_attn.so (the C-ABI HIP library) for gfx950 with hipcc, and beside it the
+measuring library csrc/probes/libpa_probes.so (csrc/probes/pa_probes.h: what bench.py times the
+kernels against; never loaded by the package).
 
-Usage:  python build.py [--force]
+Usage:  python build.py
 
 Each csrc/*.hip file is compiled to an object in csrc/_obj/ (in parallel) and the objects
-are linked into libpaged_attn.so next to this file.  hipcc cross-compiles for gfx950
-without a GPU present.  The library depends on the HIP runtime only (no torch symbols).
+are linked into libpaged_attn.so next to this file; csrc/probes/*.hip likewise into
+libpa_probes.so.  hipcc cross-compiles for gfx950 without a GPU present.  The libraries depend
+on the HIP runtime only (no torch symbols).
 """
 import concurrent.futures
 import os
@@ -17,13 +20,15 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OBJ = os.path.join(CSRC, "_obj")
 LIB = os.path.join(HERE, "libpaged_attn.so")
+PROBES = os.path.join(CSRC, "probes")
+PROBES_LIB = os.path.join(PROBES, "libpa_probes.so")
 ARCH = "gfx950"
 
 # -packed-fp32-ops: keep hipcc from forming v_pk_{add,mul,fma}_f32 out of ordinary float code.
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
             f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
-            "-I", INCLUDE, "-I", CSRC, "-Rpass-analysis=kernel-resource-usage"] + DEVICE_FLAGS
+            "-I", INCLUDE, "-I", CSRC, "-I", PROBES, "-Rpass-analysis=kernel-resource-usage"] + DEVICE_FLAGS
 
 
 def _hipcc():
@@ -37,18 +42,25 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def probe_sources():
+    return sorted(os.path.join(PROBES, f) for f in os.listdir(PROBES) if f.endswith(".hip"))
+
+
 def _newest_input():
-    files = sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    files = sources() + probe_sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    files += [os.path.join(PROBES, f) for f in os.listdir(PROBES) if f.endswith(".h")]
     files += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE)] + [os.path.abspath(__file__)]
     return max(os.path.getmtime(f) for f in files)
 
 
 def is_current():
-    return os.path.exists(LIB) and os.path.getmtime(LIB) >= _newest_input()
+    newest = _newest_input()
+    return all(os.path.exists(lib) and os.path.getmtime(lib) >= newest for lib in (LIB, PROBES_LIB))
 
 
 def _compile(hipcc, src):
-    obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+    prefix = "probes_" if os.path.dirname(src) == PROBES else ""
+    obj = os.path.join(OBJ, prefix + os.path.basename(src)[:-4] + ".o")
     cmd = [hipcc] + CXXFLAGS + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -86,19 +98,21 @@ def build_library(force=True, verbose=False):
         return LIB
     hipcc = _hipcc()
     os.makedirs(OBJ, exist_ok=True)
-    srcs = sources()
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        results = list(ex.map(lambda s: _compile(hipcc, s), srcs))
+    srcs, probes = sources(), probe_sources()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as ex:
+        results = list(ex.map(lambda s: _compile(hipcc, s), srcs + probes))
     for obj, msgs in results:
         if verbose and msgs:
             print(msgs, file=sys.stderr)
     objs = [o for o, _ in results]
-    tmp = LIB + ".tmp"
-    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", "-o", tmp] + objs
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
-    os.replace(tmp, LIB)
+    # -Bsymbolic: each library binds its own copy of the helpers both define (pa::fail, ...)
+    for lib, members in ((LIB, objs[:len(srcs)]), (PROBES_LIB, objs[len(srcs):])):
+        tmp = lib + ".tmp"
+        cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-fno-gpu-rdc", "-Wl,-Bsymbolic", "-o", tmp] + members
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+        os.replace(tmp, lib)
     return LIB
 
 

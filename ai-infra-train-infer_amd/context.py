@@ -27,8 +27,9 @@ class InferenceContext:
     # [num_seqs, max_blocks] physical block ids; entries past the context are never read
     block_tables: Optional[torch.Tensor] = None
     # decode, optional (no counterpart in the reference): rows that share prefixes as the same
-    # physical blocks, as attention.prepare_prefix_groups() returns them; None = read every row alone
-    prefix_groups: Optional[dict] = None
+    # physical blocks, as attention.prepare_prefix_groups() returns them (a PrefixGroups); None = read
+    # every row alone
+    prefix_groups: Optional[object] = None
 
 
 _CONTEXT = InferenceContext()
@@ -43,7 +44,7 @@ def set_context(
     slot_mapping: Optional[torch.Tensor] = None,
     context_lens: Optional[torch.Tensor] = None,
     block_tables: Optional[torch.Tensor] = None,
-    prefix_groups: Optional[dict] = None,
+    prefix_groups: Optional[object] = None,
 ):
     """Install the context for the next model forward."""
     global _CONTEXT

@@ -23,6 +23,6 @@ int check_launch(const char* where) {
 
 }  // namespace pa
 
-extern "C" int pa_version(void) { return 2; }
+extern "C" int pa_version(void) { return 3; }
 
 extern "C" const char* pa_last_error(void) { return pa::g_last_error; }

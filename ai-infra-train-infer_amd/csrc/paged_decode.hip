@@ -4,7 +4,7 @@
 //
 // Reference semantics: src/inference/attention.py:317-382 (single pass), :434-476 (partitioned
 // driver), :519-589 (one partition) and :591-626 (merge).
-#include "paged_decode_kernel.hpp"
+#include "paged_decode_launch.hpp"
 
 #include <stdio.h>
 
@@ -12,34 +12,100 @@
 
 namespace pa {
 
-// out = sum_p w_p out_p / sum_p w_p, w_p = sum_p * exp(max_p - max); one workgroup per
-// (query head, batch row), one thread per head-dim element.
-__global__ void merge_partitions_kernel(const float* __restrict__ ws_max,
-                                        const float* __restrict__ ws_sum,
-                                        const float* __restrict__ ws_out,
-                                        const int32_t* __restrict__ context_lens, void* out,
-                                        int out_dtype, int64_t out_stride, int num_q_heads,
-                                        int head_dim, int partition_size, int max_partitions) {
+// out = sum_p w_p out_p / sum_p w_p, w_p = sum_p * exp(max_p - max), over the partitions of one
+// (batch row, query head) per workgroup.  A partition's partial output (head_dim floats) is read
+// by head_dim / 4 lanes as 16-byte pieces, so the 256 threads of the workgroup work on several
+// partitions at once ("slots": 8 at head_dim 128), each slot taking every slots-th partition in
+// one pass with a running maximum, four independent loads in flight per thread; the slots are
+// then combined through LDS.  (Before: one thread per element walking all partitions twice, 8.9 us
+// for 53 partitions of 4 x 16 rows.)
+constexpr int kMergeThreads = 256;
+constexpr int kMergeUnroll = 4;
+
+__global__ __launch_bounds__(kMergeThreads) void merge_partitions_kernel(
+    const float* __restrict__ ws_max, const float* __restrict__ ws_sum, const float* __restrict__ ws_out,
+    const int32_t* __restrict__ context_lens, void* out, int out_dtype, int64_t out_stride, int num_q_heads,
+    int head_dim, int partition_size, int max_partitions) {
+  __shared__ float4 s_acc[kMergeThreads];
+  __shared__ float s_m[kMergeThreads], s_den[kMergeThreads];
   const int h = blockIdx.x;
   const int b = blockIdx.y;
-  const int d = threadIdx.x;
+  const int tid = threadIdx.x;
   const int ctx = context_lens[b];
-  const int64_t o = b * out_stride + (int64_t)h * head_dim + d;
+  const int64_t o = b * out_stride + (int64_t)h * head_dim;
   if (ctx <= 0) {
-    store_from_f32(out, o, out_dtype, 0.0f);
+    for (int d = tid; d < head_dim; d += kMergeThreads) store_from_f32(out, o + d, out_dtype, 0.0f);
     return;
   }
   const int np = min((ctx + partition_size - 1) / partition_size, max_partitions);
+  const int lpp = head_dim >> 2;                 // lanes per partition row
+  const int slots = kMergeThreads / lpp;
+  const int slot = tid / lpp;
+  const int ld = tid - slot * lpp;               // which 16-byte piece of the row
   const int64_t row0 = ((int64_t)b * num_q_heads + h) * max_partitions;
-  float mx = -INFINITY;
-  for (int q = 0; q < np; ++q) mx = fmaxf(mx, ws_max[row0 + q]);
-  float num = 0.0f, den = 0.0f;
-  for (int q = 0; q < np; ++q) {
-    const float w = ws_sum[row0 + q] * __expf(ws_max[row0 + q] - mx);
-    den += w;
-    num = fmaf(w, ws_out[(row0 + q) * head_dim + d], num);
+  float m = -INFINITY, den = 0.0f;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (slot < slots) {
+    for (int q0 = slot; q0 < np; q0 += slots * kMergeUnroll) {
+      float pm[kMergeUnroll], ps[kMergeUnroll];
+      float4 po[kMergeUnroll];
+#pragma unroll
+      for (int u = 0; u < kMergeUnroll; ++u) {
+        const int q = q0 + u * slots;
+        const bool live = q < np;
+        const int64_t r = row0 + (live ? q : q0);
+        pm[u] = live ? ws_max[r] : -INFINITY;
+        ps[u] = live ? ws_sum[r] : 0.0f;
+        po[u] = *(const float4*)(ws_out + r * head_dim + 4 * ld);
+      }
+#pragma unroll
+      for (int u = 0; u < kMergeUnroll; ++u) {
+        const float m_new = fmaxf(m, pm[u]);     // finite: partition q0 of this pass is live
+        const float a = __expf(m - m_new);
+        const float w = ps[u] * __expf(pm[u] - m_new);
+        den = fmaf(den, a, w);
+        acc.x = fmaf(acc.x, a, w * po[u].x);
+        acc.y = fmaf(acc.y, a, w * po[u].y);
+        acc.z = fmaf(acc.z, a, w * po[u].z);
+        acc.w = fmaf(acc.w, a, w * po[u].w);
+        m = m_new;
+      }
+    }
   }
-  store_from_f32(out, o, out_dtype, num / den);
+  s_m[tid] = m;
+  s_den[tid] = den;
+  s_acc[tid] = acc;
+  __syncthreads();
+  if (slot != 0) return;
+  const int used = min(slots, np);               // slots that saw a partition
+  float mx = m;
+  for (int i = 1; i < used; ++i) mx = fmaxf(mx, s_m[i * lpp + ld]);
+  float d_all = 0.0f;
+  float4 n_all = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (int i = 0; i < used; ++i) {
+    const int t = i * lpp + ld;
+    const float w = __expf(s_m[t] - mx);
+    const float4 a = s_acc[t];
+    d_all = fmaf(s_den[t], w, d_all);
+    n_all.x = fmaf(a.x, w, n_all.x);
+    n_all.y = fmaf(a.y, w, n_all.y);
+    n_all.z = fmaf(a.z, w, n_all.z);
+    n_all.w = fmaf(a.w, w, n_all.w);
+  }
+  const float inv = 1.0f / d_all;
+  store_from_f32(out, o + 4 * ld, out_dtype, n_all.x * inv);
+  store_from_f32(out, o + 4 * ld + 1, out_dtype, n_all.y * inv);
+  store_from_f32(out, o + 4 * ld + 2, out_dtype, n_all.z * inv);
+  store_from_f32(out, o + 4 * ld + 3, out_dtype, n_all.w * inv);
+}
+
+static int launch_merge(const float* ws_max, const float* ws_sum, const float* ws_out, const int32_t* context_lens,
+                        void* out, int out_dtype, int64_t out_stride, int64_t batch, int64_t num_q_heads,
+                        int64_t head_dim, int64_t partition_size, int64_t max_partitions, hipStream_t st) {
+  hipLaunchKernelGGL(merge_partitions_kernel, dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kMergeThreads), 0,
+                     st, ws_max, ws_sum, ws_out, context_lens, out, out_dtype, out_stride, (int)num_q_heads,
+                     (int)head_dim, (int)partition_size, (int)max_partitions);
+  return PA_OK;
 }
 
 // Debug aid: counts what the attention kernels would silently clamp.  counts[0] = block-table
@@ -62,82 +128,59 @@ __global__ void check_tables_kernel(const int32_t* __restrict__ block_tables, in
 // Debug aid for shared-prefix launches: counts[0] = table entries of a group's shared partitions
 // that differ between a row and the group's first row; counts[1] = rows whose context is shorter
 // than the tokens their group shares, or whose row_skip differs from their group's shared
-// partitions; counts[2] = rows that belong to no group but have a non-zero row_skip, or to two groups.
+// partitions, and groups that reach outside the batch or the row list; counts[2] = rows that belong
+// to no group but have a non-zero row_skip, or to two groups.
 // One workgroup per group, one thread per shared table entry (strided).
 __global__ void check_shared_prefix_kernel(const int32_t* __restrict__ block_tables, int64_t bt_stride,
                                            int table_width, const int32_t* __restrict__ context_lens,
                                            int batch, int bs_log2, int partition_size,
                                            const int32_t* __restrict__ group_desc, int num_groups,
+                                           const int32_t* __restrict__ group_rows, int group_rows_len,
                                            const int32_t* __restrict__ row_skip, int32_t* counts) {
   const int gi = blockIdx.x;
+  auto row_of = [&](int k, int m) { return group_rows ? group_rows[group_desc[4 * k] + m] : group_desc[4 * k] + m; };
+  auto well_formed = [&](int k) {
+    const int first = group_desc[4 * k], rows = group_desc[4 * k + 1];
+    if (rows < 1 || first < 0 || group_desc[4 * k + 2] < 0) return false;
+    return group_rows ? first + rows <= group_rows_len : first + rows <= batch;
+  };
   if (gi == num_groups) {
     // rows outside every group must skip nothing; rows inside exactly one
     for (int b = threadIdx.x; b < batch; b += blockDim.x) {
       int owners = 0;
-      for (int k = 0; k < num_groups; ++k)
-        owners += (b >= group_desc[4 * k] && b < group_desc[4 * k] + group_desc[4 * k + 1]) ? 1 : 0;
+      for (int k = 0; k < num_groups; ++k) {
+        if (!well_formed(k) || group_desc[4 * k + 2] == 0) continue;      // empty groups claim nothing
+        for (int m = 0; m < group_desc[4 * k + 1]; ++m) owners += row_of(k, m) == b ? 1 : 0;
+      }
       if ((owners == 0 && row_skip[b] != 0) || owners > 1) atomicAdd(&counts[2], 1);
     }
     return;
   }
-  const int first = group_desc[4 * gi], rows = group_desc[4 * gi + 1], parts = group_desc[4 * gi + 2];
+  const int rows = group_desc[4 * gi + 1], parts = group_desc[4 * gi + 2];
+  if (parts == 0) return;                                                   // an empty (padding) group
   const int shared_tokens = parts * partition_size;
   const int shared_blocks = (shared_tokens + (1 << bs_log2) - 1) >> bs_log2;
-  if (first < 0 || rows < 1 || first + rows > batch || parts < 0) {
+  if (!well_formed(gi)) {
     if (threadIdx.x == 0) atomicAdd(&counts[1], 1);
     return;
   }
-  for (int m = threadIdx.x; m < rows; m += blockDim.x)
-    if (context_lens[first + m] < shared_tokens || row_skip[first + m] != parts) atomicAdd(&counts[1], 1);
+  for (int m = 0; m < rows; ++m) {
+    const int r = row_of(gi, m);
+    if (r < 0 || r >= batch) {
+      if (threadIdx.x == 0) atomicAdd(&counts[1], 1);
+      return;
+    }
+  }
+  const int lead = row_of(gi, 0);
+  for (int m = threadIdx.x; m < rows; m += blockDim.x) {
+    const int r = row_of(gi, m);
+    if (context_lens[r] < shared_tokens || row_skip[r] != parts) atomicAdd(&counts[1], 1);
+  }
   for (int e = threadIdx.x; e < shared_blocks * (rows - 1); e += blockDim.x) {
     const int m = 1 + e / shared_blocks, c = e % shared_blocks;
-    if (c >= table_width || block_tables[(first + m) * bt_stride + c] != block_tables[first * bt_stride + c])
+    if (c >= table_width || block_tables[row_of(gi, m) * bt_stride + c] != block_tables[lead * bt_stride + c])
       atomicAdd(&counts[0], 1);
   }
-}
-
-// CUs of the current device (per device, asked once).
-static int compute_units() {
-  static int cached[kMaxDevices] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-  int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
-  }
-  return n;
-}
-
-struct Workspace {
-  float* mx;
-  float* sum;
-  float* out;
-};
-
-static int64_t ws_bytes(int64_t batch, int64_t hq, int64_t d, int64_t maxp) {
-  if (maxp < 1) maxp = 1;
-  const int64_t rows = batch * hq * maxp;
-  // max and sum are padded to a 256-byte boundary so the partial outputs stay 16-byte aligned
-  const int64_t scalars = ((rows * 4 + 255) / 256) * 256;
-  return 2 * scalars + rows * d * 4;
-}
-
-static Workspace ws_split(void* ws, int64_t batch, int64_t hq, int64_t maxp) {
-  const int64_t rows = batch * hq * maxp;
-  const int64_t scalars = ((rows * 4 + 255) / 256) * 256;
-  Workspace w;
-  w.mx = (float*)ws;
-  w.sum = (float*)((uint8_t*)ws + scalars);
-  w.out = (float*)((uint8_t*)ws + 2 * scalars);
-  return w;
-}
-
-static int ilog2_exact(int64_t v) {
-  if (v <= 0 || (v & (v - 1)) != 0) return -1;
-  int l = 0;
-  while ((int64_t(1) << l) < v) ++l;
-  return l;
 }
 
 // ---- scratch of the entry point that allocates nothing ------------------------------------------
@@ -171,22 +214,9 @@ static int scratch_for_current_device(void** out) {
   return PA_OK;
 }
 
-enum { kDecodeFull = 0, kDecodePartials = 1, kDecodeProbe = 2 };
+enum { kDecodeFull = 0, kDecodePartials = 1 };
 
-// What pa_decode_shared_prefix adds to a partitioned launch.
-struct SharedPrefix {
-  const int32_t* group_desc;
-  int64_t num_groups;
-  int64_t max_group_rows;
-  int64_t max_shared_partitions;
-  const int32_t* row_skip;
-  int64_t max_own_partitions;
-};
-
-constexpr int kMatrixPath = 16;            // q_heads_per_wave value that names the MFMA kernel
-constexpr int kMatrixPathFromRatio = 3;     // GQA ratio from which the automatic choice takes it
-
-// Shared argument checking + launch of the attention pass; `merge` adds the reduction.
+// Shared argument checking + launch of the attention pass; kDecodeFull adds the reduction.
 static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_token_stride,
                        const void* k_cache, const void* v_cache, const float* k_scale,
                        const float* v_scale, int kv_dtype, const int32_t* block_tables,
@@ -198,225 +228,25 @@ static int decode_impl(const char* who, const void* q, int q_dtype, int64_t q_to
                        int waves, int kv_heads_per_wave, int q_heads_per_wave, int mode,
                        void* stream, const SharedPrefix* shared = nullptr) {
   const bool merge = mode == kDecodeFull;
-  char msg[256];
-#define PA_FAIL(code, text)                         \
-  do {                                              \
-    snprintf(msg, sizeof(msg), "%s: %s", who, text); \
-    return fail(code, msg);                         \
-  } while (0)
-  if (batch < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
-      num_blocks <= 0 || bt_stride < 0 || table_width < 0)
-    PA_FAIL(PA_ERR_BAD_ARG, "negative or zero size");
-  if (batch == 0) return PA_OK;
-  if (!q || !k_cache || !v_cache || !block_tables || !context_lens)
-    PA_FAIL(PA_ERR_BAD_ARG, "null pointer");
-  if (merge && !out) PA_FAIL(PA_ERR_BAD_ARG, "null output");
-  if (table_width > bt_stride && batch > 1) PA_FAIL(PA_ERR_BAD_ARG, "table_width larger than the row stride");
-  if (table_width > 0x7fffffff) PA_FAIL(PA_ERR_BAD_ARG, "table_width too large");
-  if (q_dtype != PA_DTYPE_F16 && q_dtype != PA_DTYPE_BF16 && q_dtype != PA_DTYPE_F32)
-    PA_FAIL(PA_ERR_UNSUPPORTED, "q_dtype must be f16, bf16 or f32");
-  int kv;
-  switch (kv_dtype) {
-    case PA_DTYPE_F16: kv = KV_F16; break;
-    case PA_DTYPE_BF16: kv = KV_BF16; break;
-    case PA_DTYPE_FP8_E4M3: kv = KV_FP8; break;
-    default: PA_FAIL(PA_ERR_UNSUPPORTED, "kv_dtype must be f16, bf16 or fp8-e4m3");
-  }
-  if (kv == KV_FP8 && (!k_scale || !v_scale))
-    PA_FAIL(PA_ERR_BAD_ARG, "fp8 cache needs k_scale and v_scale");
-  if (kv == KV_FP8 && (!aligned16(k_scale) || !aligned16(v_scale)))
-    PA_FAIL(PA_ERR_BAD_ARG, "k_scale and v_scale must be 16-byte aligned");
-  if (head_dim != 64 && head_dim != 128) PA_FAIL(PA_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
-  if (num_q_heads % num_kv_heads != 0)
-    PA_FAIL(PA_ERR_BAD_ARG, "num_q_heads must be a multiple of num_kv_heads");
-  const int bs_log2 = ilog2_exact(block_size);
-  if (bs_log2 < 3) PA_FAIL(PA_ERR_UNSUPPORTED, "block_size must be a power of two >= 8");
-  if (!aligned16(k_cache) || !aligned16(v_cache))
-    PA_FAIL(PA_ERR_BAD_ARG, "caches must be 16-byte aligned");
-  if (q_token_stride < num_q_heads * head_dim || (out && out_token_stride < num_q_heads * head_dim))
-    PA_FAIL(PA_ERR_BAD_ARG, "token stride smaller than num_q_heads*head_dim");
-  if (batch > 65535 || num_blocks > 0x7fffffff || num_q_heads > 65535)
-    PA_FAIL(PA_ERR_UNSUPPORTED, "batch or head count too large for one launch");
-  if (max_partitions < 1) max_partitions = 1;
-  if (max_partitions > 65535) PA_FAIL(PA_ERR_UNSUPPORTED, "max_partitions > 65535");
-  if (waves != 0 && waves != 1 && waves != 2 && waves != 4 && waves != 8)
-    PA_FAIL(PA_ERR_BAD_ARG, "waves_per_workgroup must be 0 (automatic), 1, 2, 4 or 8");
-  if (kv_heads_per_wave != 0 && kv_heads_per_wave != 1 && kv_heads_per_wave != 2 &&
-      kv_heads_per_wave != 4 && kv_heads_per_wave != 8)
-    PA_FAIL(PA_ERR_BAD_ARG, "kv_heads_per_wave must be 0 (automatic), 1, 2, 4 or 8");
-  if (q_heads_per_wave != 0 && q_heads_per_wave != 1 && q_heads_per_wave != 2 && q_heads_per_wave != 4 &&
-      q_heads_per_wave != kMatrixPath)
-    PA_FAIL(PA_ERR_BAD_ARG, "q_heads_per_wave must be 0 (automatic), 1, 2, 4 or 16 (the matrix path)");
-  const bool direct = merge && max_partitions == 1 && !shared;
-  if (shared) {
-    if (!shared->group_desc || !shared->row_skip) PA_FAIL(PA_ERR_BAD_ARG, "null group descriptors");
-    if (shared->num_groups < 0 || shared->num_groups > 0x7fffffff || shared->max_group_rows < 1 ||
-        shared->max_shared_partitions < 0 || shared->max_shared_partitions > max_partitions ||
-        shared->max_own_partitions < 1 || shared->max_own_partitions > max_partitions)
-      PA_FAIL(PA_ERR_BAD_ARG, "group counts out of range");
-    if (partition_size <= 0) PA_FAIL(PA_ERR_BAD_ARG, "a shared-prefix launch is a partitioned launch: partition_size > 0");
-    if ((num_q_heads / num_kv_heads) * shared->max_group_rows > kMatrixPath)
-      PA_FAIL(PA_ERR_UNSUPPORTED, "rows per group x query heads per KV head must not exceed 16");
-    if (kv_heads_per_wave > 1 || (q_heads_per_wave != 0 && q_heads_per_wave != kMatrixPath) || waves == 1)
-      PA_FAIL(PA_ERR_UNSUPPORTED, "a shared-prefix launch runs on the matrix path with one KV head per wave");
-  }
-  if (!direct) {
-    if ((max_partitions > 1 || shared) && (partition_size <= 0 || partition_size % 16 != 0))
-      PA_FAIL(PA_ERR_UNSUPPORTED, "partition_size must be a positive multiple of 16");
-    const int64_t need = ws_bytes(batch, num_q_heads, head_dim, max_partitions);
-    if (!workspace || workspace_bytes < need) PA_FAIL(PA_ERR_WORKSPACE, "workspace missing or too small");
-    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
-      PA_FAIL(PA_ERR_BAD_ARG, "workspace must be 256-byte aligned");
-    if (partition_size > 0x7fffffff) PA_FAIL(PA_ERR_BAD_ARG, "partition_size too large");
-  }
-
-  // ---- how the query group of a KV head is spread over registers, waves and workgroups ----------
-  // gc query heads in a wave's registers; qs groups of waves over the same tokens when the group
-  // is wider than that; whatever is left over (ratios with a factor other than 2) goes to
-  // separate workgroups, which then read the KV head once each.
-  const int g = (int)(num_q_heads / num_kv_heads);
-  DecodeShape s;
-  s.head_dim = (int)head_dim;
-  int slices;                                 // workgroups per KV head
-  // The matrix path (paged_decode_mfma_kernel.hpp) takes up to 16 query heads of a KV head as one
-  // MFMA operand: the choice from a GQA ratio of 3 on, where the vector kernel's arithmetic per
-  // loaded byte starts to cost more than the loads (batch 64 x 4096 tokens, fp16 / fp8 cache: ratio 4
-  // 187 / 103 us against 195 / 142 us, ratio 8 187 / 103 against 239 / 257, ratio 2 182 / 100.5 against 179 / 100).
-  bool matrix = q_heads_per_wave == kMatrixPath || shared != nullptr;
-  if (q_heads_per_wave == 0 && g >= kMatrixPathFromRatio && mode != kDecodeProbe && kv_heads_per_wave <= 2 &&
-      (waves == 0 || waves >= 2) && !(kv_heads_per_wave == 2 && (waves == 8 || num_kv_heads % 2 != 0)))
-    matrix = true;
-  if (matrix) {
-    if (mode == kDecodeProbe) PA_FAIL(PA_ERR_UNSUPPORTED, "the load probe follows the vector kernel: q_heads_per_wave 1, 2 or 4");
-    if (kv_heads_per_wave > 2 || (kv_heads_per_wave == 2 && num_kv_heads % 2 != 0))
-      PA_FAIL(PA_ERR_UNSUPPORTED, "the matrix path takes one KV head per wave, or two of an even number");
-    if (waves == 1 || (kv_heads_per_wave == 2 && waves == 8))
-      PA_FAIL(PA_ERR_UNSUPPORTED, "the matrix path takes 2, 4 or 8 waves per workgroup with one KV head per wave, 2 or 4 with two");
-    s.gc = kMatrixPath;
-    s.qs = 1;
-    slices = (g + kMatrixPath - 1) / kMatrixPath;
-    // One KV head per wave.  4-wave workgroups (two share a CU) are the best or within 3 % of the best
-    // shape from batch 8 x 320 to batch 256 x 1k tokens; launches with fewer workgroups than CUs put
-    // 8 waves on the CUs they do reach.  Two heads per wave (256-byte pieces of an fp8 row, 32 KiB of
-    // LDS per wave, so one 4-wave workgroup per CU) pay in one case only: an fp8 cache and a halved
-    // grid that is just one workgroup per CU (batch 64 x 8 KV heads: 103-105 against 112-115 us);
-    // with fewer workgroups they idle CUs, with more the second round costs what the pieces save.
-    s.hpw = kv_heads_per_wave == 2 ? 2 : 1;
-    const int64_t cus = compute_units();
-    const int64_t unpaired = num_kv_heads * slices * max_partitions * batch;
-    if (kv_heads_per_wave == 0 && kv == KV_FP8 && num_kv_heads % 2 == 0 && !shared && (waves == 0 || waves == 4) &&
-        unpaired / 2 <= cus && unpaired / 2 * 10 >= cus * 9)
-      s.hpw = 2;
-    if (waves != 0) {
-      s.waves = waves;
-    } else {
-      s.waves = (s.hpw == 1 && unpaired < cus && !shared) ? 8 : 4;
-    }
-  } else {
-    if (q_heads_per_wave != 0) {
-      if (g % q_heads_per_wave != 0) PA_FAIL(PA_ERR_UNSUPPORTED, "q_heads_per_wave must divide num_q_heads / num_kv_heads");
-      s.gc = q_heads_per_wave;
-    } else {
-      s.gc = (g % 4 == 0) ? 4 : (g % 2 == 0) ? 2 : 1;
-    }
-    const int rest = g / s.gc;
-    const int split_waves = s.gc == 4 ? 4 : 8;
-    s.qs = 1;
-    if (s.gc >= 2 && rest % 2 == 0 && (waves == 0 || waves == split_waves)) s.qs = (rest % 4 == 0) ? 4 : 2;
-    slices = rest / s.qs;
-    s.waves = s.qs > 1 ? split_waves : (waves == 0 ? 4 : waves);
-    // Several adjacent KV heads per wave need each KV head's query group whole in the wave.
-    const bool can_share = g == s.gc && s.gc <= 2;
-    s.hpw = 1;
-    if (kv_heads_per_wave > 1) {
-      if (!can_share || num_kv_heads % kv_heads_per_wave != 0 ||
-          (kv_heads_per_wave > 2 && (s.gc != 2 || (s.waves != 4 && s.waves != 8))))
-        PA_FAIL(PA_ERR_UNSUPPORTED, "kv_heads_per_wave does not fit this head layout");
-      s.hpw = kv_heads_per_wave;
-    } else if (kv_heads_per_wave == 0 && can_share && num_kv_heads % 2 == 0) {
-      // Two heads per wave when halving the workgroups does not add a round of them over the CUs: a
-      // CU streams at a fixed rate however many workgroups it hosts, the launch takes as long as
-      // its busiest CU, and fewer, longer-lived workgroups stream better (185 -> 178 us at batch 64 /
-      // ctx 4096, fp16; rows of 128 bytes or less gain another 10% from being read as 256-byte
-      // pieces).  With a workgroup or less per CU pairing would only idle CUs.
-      const int64_t cus = compute_units();
-      const int64_t wgs = num_kv_heads * max_partitions * batch;      // unpaired
-      const int64_t rounds = (wgs + cus - 1) / cus, paired_rounds = (wgs + 2 * cus - 1) / (2 * cus);
-      if (wgs >= 8 * cus || 2 * paired_rounds <= rounds) s.hpw = 2;
-    }
-  }
-#undef PA_FAIL
-
-  DecodeParams p;
-  p.q = q;
-  p.q_stride = q_token_stride;
-  p.k_cache = (const uint8_t*)k_cache;
-  p.v_cache = (const uint8_t*)v_cache;
-  p.k_scale = k_scale;
-  p.v_scale = v_scale;
-  p.block_tables = block_tables;
-  p.bt_stride = bt_stride;
-  p.table_width = (int)table_width;
-  p.context_lens = context_lens;
-  p.out = out;
-  p.out_stride = out_token_stride;
-  p.q_dtype = q_dtype;
-  p.num_q_heads = (int)num_q_heads;
-  p.num_kv_heads = (int)num_kv_heads;
-  p.bs_log2 = bs_log2;
-  p.num_blocks = (int)num_blocks;
-  p.partition_size = (int)partition_size;
-  p.max_partitions = (int)max_partitions;
-  p.direct_out = direct ? 1 : 0;
-  p.scale_log2e = scale * 1.4426950408889634f;
-  p.ws_max = p.ws_sum = p.ws_out = nullptr;
-  if (!direct) {
-    const Workspace w = ws_split(workspace, batch, num_q_heads, max_partitions);
-    p.ws_max = w.mx;
-    p.ws_sum = w.sum;
-    p.ws_out = w.out;
-  }
-
+  DecodePlan plan;
+  int rc = plan_decode(who, q, q_dtype, q_token_stride, k_cache, v_cache, k_scale, v_scale, kv_dtype,
+                       block_tables, bt_stride, table_width, context_lens, out, out_token_stride, batch,
+                       num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, partition_size,
+                       max_partitions, workspace, workspace_bytes, waves, kv_heads_per_wave,
+                       q_heads_per_wave, merge, false, shared, &plan);
+  if (rc != PA_OK || plan.empty) return rc;
   hipStream_t st = (hipStream_t)stream;
-  p.inner = (int)(num_kv_heads / s.hpw) * slices;
-  p.probe = mode == kDecodeProbe ? 1 : 0;
-  p.batch = (int)batch;
-  p.group_desc = nullptr;
-  p.row_skip = nullptr;
-  p.num_prefix_wgs = p.prefix_parts = p.suffix_parts = 0;
-  int64_t wgs = batch * max_partitions * p.inner;
-  if (shared) {
-    const int64_t prefix_wgs = shared->num_groups * shared->max_shared_partitions * p.inner;
-    wgs = prefix_wgs + batch * shared->max_own_partitions * p.inner;
-    if (prefix_wgs > 0x7fffffff) {
-      snprintf(msg, sizeof(msg), "%s: too many workgroups for one launch", who);
-      return fail(PA_ERR_UNSUPPORTED, msg);
-    }
-    p.group_desc = shared->group_desc;
-    p.row_skip = shared->row_skip;
-    p.num_prefix_wgs = (int)prefix_wgs;
-    p.prefix_parts = (int)shared->max_shared_partitions;
-    p.suffix_parts = (int)shared->max_own_partitions;
-  }
-  if (wgs > 0x7fffffff) {
-    snprintf(msg, sizeof(msg), "%s: too many workgroups for one launch", who);
-    return fail(PA_ERR_UNSUPPORTED, msg);
-  }
-  dim3 grid((unsigned)wgs);
-  int rc;
-  switch (kv) {
-    case KV_F16: rc = launch_decode_f16(p, grid, s, st); break;
-    case KV_BF16: rc = launch_decode_bf16(p, grid, s, st); break;
-    default: rc = launch_decode_fp8(p, grid, s, st); break;
+  const dim3 grid(plan.grid);
+  switch (plan.kv) {
+    case KV_F16: rc = launch_decode_f16(plan.p, grid, plan.s, st); break;
+    case KV_BF16: rc = launch_decode_bf16(plan.p, grid, plan.s, st); break;
+    default: rc = launch_decode_fp8(plan.p, grid, plan.s, st); break;
   }
   if (rc != PA_OK) return rc;
   rc = check_launch(who);
-  if (rc != PA_OK || direct || !merge) return rc;
-
-  hipLaunchKernelGGL(merge_partitions_kernel, dim3((unsigned)num_q_heads, (unsigned)batch),
-                     dim3((unsigned)head_dim), 0, st, p.ws_max, p.ws_sum, p.ws_out, context_lens,
-                     out, q_dtype, out_token_stride, (int)num_q_heads, (int)head_dim,
-                     (int)partition_size, (int)max_partitions);
+  if (rc != PA_OK || plan.direct || !merge) return rc;
+  launch_merge(plan.p.ws_max, plan.p.ws_sum, plan.p.ws_out, context_lens, out, q_dtype, out_token_stride, batch,
+               num_q_heads, head_dim, plan.p.partition_size, plan.p.max_partitions, st);
   return check_launch(who);
 }
 
@@ -507,11 +337,14 @@ extern "C" int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_tok
                                        int64_t num_blocks, float scale, int64_t partition_size,
                                        int64_t max_partitions, void* workspace, int64_t workspace_bytes,
                                        int waves_per_workgroup, const int32_t* group_desc,
-                                       int64_t num_groups, int64_t max_group_rows,
+                                       int64_t num_groups, const int32_t* group_rows,
+                                       int64_t num_group_rows, int64_t max_group_rows,
                                        int64_t max_shared_partitions, const int32_t* row_skip,
                                        int64_t max_own_partitions, void* stream) {
-  const SharedPrefix sp = {group_desc, num_groups, max_group_rows, max_shared_partitions, row_skip,
-                           max_own_partitions};
+  if (group_rows && (num_group_rows < 0 || num_group_rows > 0x7fffffff))
+    return fail(PA_ERR_BAD_ARG, "pa_decode_shared_prefix: num_group_rows out of range");
+  const SharedPrefix sp = {group_desc, group_rows, group_rows ? num_group_rows : 0, num_groups, max_group_rows,
+                           max_shared_partitions, row_skip, max_own_partitions};
   return decode_impl("pa_decode_shared_prefix", q, q_dtype, q_token_stride, k_cache, v_cache, k_scale,
                      v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, out,
                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim, block_size,
@@ -522,7 +355,8 @@ extern "C" int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_tok
 extern "C" int pa_check_shared_prefix(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
                                       const int32_t* context_lens, int64_t batch, int64_t block_size,
                                       int64_t partition_size, const int32_t* group_desc,
-                                      int64_t num_groups, const int32_t* row_skip, int32_t* counts,
+                                      int64_t num_groups, const int32_t* group_rows,
+                                      int64_t num_group_rows, const int32_t* row_skip, int32_t* counts,
                                       void* stream) {
   if (batch < 0 || bt_stride < 0 || table_width < 0 || num_groups < 0 || partition_size <= 0)
     return fail(PA_ERR_BAD_ARG, "pa_check_shared_prefix: negative or zero size");
@@ -532,11 +366,13 @@ extern "C" int pa_check_shared_prefix(const int32_t* block_tables, int64_t bt_st
   if (batch == 0) return PA_OK;
   if (!block_tables || !context_lens || !row_skip || (num_groups > 0 && !group_desc))
     return fail(PA_ERR_BAD_ARG, "pa_check_shared_prefix: null pointer");
-  if (batch > 0x7fffffff || table_width > 0x7fffffff || num_groups >= 0x7fffffff || partition_size > 0x7fffffff)
+  if (batch > 0x7fffffff || table_width > 0x7fffffff || num_groups >= 0x7fffffff || partition_size > 0x7fffffff ||
+      num_group_rows < 0 || num_group_rows > 0x7fffffff)
     return fail(PA_ERR_UNSUPPORTED, "pa_check_shared_prefix: batch, table or group count too large for one launch");
   hipLaunchKernelGGL(check_shared_prefix_kernel, dim3((unsigned)num_groups + 1), dim3(256), 0,
                      (hipStream_t)stream, block_tables, bt_stride, (int)table_width, context_lens,
-                     (int)batch, bs_log2, (int)partition_size, group_desc, (int)num_groups, row_skip, counts);
+                     (int)batch, bs_log2, (int)partition_size, group_desc, (int)num_groups, group_rows,
+                     group_rows ? (int)num_group_rows : 0, row_skip, counts);
   return check_launch("pa_check_shared_prefix");
 }
 
@@ -548,34 +384,19 @@ extern "C" int pa_merge(const void* workspace, int64_t workspace_bytes, const in
     return fail(PA_ERR_BAD_ARG, "pa_merge: bad size");
   if (batch == 0) return PA_OK;
   if (!workspace || !context_lens || !out) return fail(PA_ERR_BAD_ARG, "pa_merge: null pointer");
-  if (head_dim > 1024) return fail(PA_ERR_UNSUPPORTED, "pa_merge: head_dim > 1024");
+  if (head_dim > 1024 || head_dim % 4 != 0) return fail(PA_ERR_UNSUPPORTED, "pa_merge: head_dim must be a multiple of 4, at most 1024");
+  if (num_q_heads > 65535 || max_partitions > 0x7fffffff || partition_size > 0x7fffffff)
+    return fail(PA_ERR_UNSUPPORTED, "pa_merge: head count, partition count or partition size too large");
   if (out_dtype != PA_DTYPE_F16 && out_dtype != PA_DTYPE_BF16 && out_dtype != PA_DTYPE_F32)
     return fail(PA_ERR_UNSUPPORTED, "pa_merge: out_dtype must be f16, bf16 or f32");
   if (workspace_bytes < ws_bytes(batch, num_q_heads, head_dim, max_partitions))
     return fail(PA_ERR_WORKSPACE, "pa_merge: workspace too small");
+  if (!aligned16(workspace)) return fail(PA_ERR_BAD_ARG, "pa_merge: workspace must be 16-byte aligned");
   if (batch > 65535) return fail(PA_ERR_UNSUPPORTED, "pa_merge: batch too large");
   const Workspace w = ws_split(const_cast<void*>(workspace), batch, num_q_heads, max_partitions);
-  hipLaunchKernelGGL(merge_partitions_kernel, dim3((unsigned)num_q_heads, (unsigned)batch),
-                     dim3((unsigned)head_dim), 0, (hipStream_t)stream, w.mx, w.sum, w.out,
-                     context_lens, out, out_dtype, out_token_stride, (int)num_q_heads,
-                     (int)head_dim, (int)partition_size, (int)max_partitions);
+  launch_merge(w.mx, w.sum, w.out, context_lens, out, out_dtype, out_token_stride, batch, num_q_heads, head_dim,
+               partition_size, max_partitions, (hipStream_t)stream);
   return check_launch("pa_merge");
-}
-
-extern "C" int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride,
-                                    const void* k_cache, const void* v_cache, const float* k_scale,
-                                    const float* v_scale, int kv_dtype, const int32_t* block_tables,
-                                    int64_t bt_stride, int64_t table_width, const int32_t* context_lens,
-                                    int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
-                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                                    int64_t partition_size, int64_t max_partitions, void* workspace,
-                                    int64_t workspace_bytes, int waves_per_workgroup,
-                                    int kv_heads_per_wave, int q_heads_per_wave, void* stream) {
-  return decode_impl("pa_decode_load_probe", q, q_dtype, q_token_stride, k_cache, v_cache, k_scale,
-                     v_scale, kv_dtype, block_tables, bt_stride, table_width, context_lens, nullptr,
-                     0, batch, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, 1.0f,
-                     partition_size, max_partitions, workspace, workspace_bytes,
-                     waves_per_workgroup, kv_heads_per_wave, q_heads_per_wave, kDecodeProbe, stream);
 }
 
 extern "C" int pa_check_tables(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,

@@ -67,7 +67,6 @@ struct DecodeParams {
   int max_partitions;
   int direct_out;
   int inner;        // workgroups per (batch row, partition): KV head groups x slices of the query group
-  int probe;        // 1: loads only, the arithmetic replaced by a checksum (pa_decode_load_probe)
   int batch;        // rows of the block table (a row's neighbours are looked at for shared blocks)
   float scale_log2e;
   // Shared prefixes (matrix kernel only; group_desc == nullptr: off).  Rows come in groups of
@@ -75,7 +74,9 @@ struct DecodeParams {
   // physical blocks: those partitions are computed once per group, by the first num_prefix_wgs
   // workgroups, for all the group's rows at once; the other workgroups take every row's own
   // partitions from row_skip[row] on.
-  const int32_t* group_desc;   // [groups][4]: first row, rows, shared partitions, unused
+  const int32_t* group_desc;   // [groups][4]: first row (or first entry of group_rows), rows, shared partitions, unused
+  const int32_t* group_rows;   // batch rows of the groups, one run per group; nullptr: a group's rows are consecutive
+  int group_rows_len;          // entries of group_rows
   const int32_t* row_skip;     // [batch]: leading partitions of the row that its group computes
   int num_prefix_wgs;          // groups x prefix_parts x inner
   int prefix_parts;            // most shared partitions of any group
@@ -207,7 +208,10 @@ struct Tile {
 // W waves per workgroup in QS groups of WQ = W / QS.  Lane layout inside a wave: lane = 8 g + j,
 // j the 16-byte piece of a row, g the row group; hs = g % HPW picks the KV head, tr = g / HPW
 // the token of a row load.
-template <int KV, int D, int GC, int W, int HPW, int QS>
+// LOADS_ONLY (a measuring build, never instantiated by the library itself): every load of the
+// launch is issued and every loaded word consumed, but the attention arithmetic is replaced by a
+// checksum, so the launch lasts as long as the memory system needs for this access pattern.
+template <int KV, int D, int GC, int W, int HPW, int QS, bool LOADS_ONLY = false>
 __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams p) {
   using G = Geo<KV, D, HPW>;
   using TileT = Tile<KV, D, HPW>;
@@ -380,8 +384,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
 
   auto consume = [&](TileT& t, int tile, auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
-    if (p.probe) {
-      // timing aid: every loaded word is used, none of the attention arithmetic is done
+    if constexpr (LOADS_ONLY) {
       uint32_t x = 0;
 #pragma unroll
       for (int r = 0; r < RL; ++r) {
@@ -392,8 +395,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
       acc[0][0] += __uint_as_float(x & 0x3fffffffu);
       l[0] = 1.0f;
       m[0] = 0.0f;
-      return;
-    }
+    } else {
     float s[RL][GC];
     bool valid[RL];
 #pragma unroll
@@ -465,6 +467,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
 #pragma unroll
         for (int k = 0; k < EPL; ++k) acc[h][k] = fmaf(pv, vf[k], acc[h][k]);
       }
+    }
     }
   };
 
@@ -594,10 +597,10 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
 
 constexpr int kMaxDevices = 64;
 
-template <int KV, int D, int GC, int W, int HPW, int QS>
+template <int KV, int D, int GC, int W, int HPW, int QS, bool LOADS_ONLY = false>
 static int launch_decode_one(const DecodeParams& p, dim3 grid, hipStream_t st) {
   constexpr int smem = decode_lds_bytes(W, GC, HPW, QS, D);
-  auto kern = paged_decode_kernel<KV, D, GC, W, HPW, QS>;
+  auto kern = paged_decode_kernel<KV, D, GC, W, HPW, QS, LOADS_ONLY>;
   if constexpr (smem > 48 * 1024) {
     // above the default dynamic LDS limit: raise it once per instantiation and device
     static bool attr_set[kMaxDevices] = {};

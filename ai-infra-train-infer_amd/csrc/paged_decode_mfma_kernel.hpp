@@ -13,10 +13,11 @@
 //  * Loads are those of the vector kernel: 16 bytes per lane, the 8 lanes of a token row read one
 //    contiguous piece, one register tile (32 tokens of K and of V) in flight per wave;
 //    non-temporal unless a neighbouring row maps the same blocks.
-//  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16; fp8 bytes
-//    are exact in fp16, their per-token scales go to LDS beside the tile and are applied to the
-//    scores and the probabilities after the products) to the wave's own 2 x 32 x head_dim fp16 of
-//    LDS, and the next tile's loads are issued into the freed registers before the products start.
+//  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16: K bytes of
+//    an fp8 cache as they are - exact in fp16 - with 1 / k_scale of the tile's tokens beside the tile
+//    in LDS and applied to the scores after the first product, V dequantised with 1 / v_scale on the
+//    way in) to the wave's own 2 x 32 x head_dim fp16 of LDS, and the next tile's loads are issued
+//    into the freed registers before the products start.
 //  * S^T = K . Q^T with v_mfma_f32_16x16x32_f16: A = 16 keys x 32 dims read back with
 //    ds_read_b128, B = Q^T (16 head columns, zero beyond the group) kept in registers, pre-scaled
 //    by scale*log2(e) and, for 16-bit caches, split into two fp16 parts (hi + lo, two products per
@@ -54,9 +55,9 @@ __device__ __forceinline__ constexpr int lds_swz(int row) {
 
 // K and V tile of one KV head
 __host__ __device__ constexpr int decode_mfma_tile_bytes(int D) { return 2 * kMfmaTile * D * 2; }
-// per wave: its tiles, then 1 / scale of the tile's 32 tokens for K and for V (fp8 caches)
+// per wave: its tiles, then 1 / k_scale of the tile's 32 tokens (fp8 caches)
 __host__ __device__ constexpr int decode_mfma_wave_bytes(int HPW, int D) {
-  return HPW * decode_mfma_tile_bytes(D) + 2 * kMfmaTile * 4;
+  return HPW * decode_mfma_tile_bytes(D) + kMfmaTile * 4;
 }
 __host__ __device__ constexpr int decode_mfma_lds_bytes(int W, int HPW, int D) {
   return W * decode_mfma_wave_bytes(HPW, D) + 2 * HPW * kMfmaHeads * W * 4;
@@ -101,6 +102,27 @@ __device__ __forceinline__ mhalf8_t words_to_f16(const uint32_t* w) {
   return r;
 }
 
+// 8 fp8 bytes (2 dwords) times a per-token factor -> 8 fp16: byte * f = byte * m * 2^e with m in
+// [1, 2); v_cvt_scalef32_pk_f16_fp8 applies the power of two exactly while it converts a pair (it
+// uses only the exponent of its scale operand) and the mantissa is one packed fp16 multiply per pair.
+__device__ __forceinline__ mhalf8_t fp8_words_to_f16_scaled(const uint32_t* w, float factor) {
+  const uint32_t bits = __float_as_uint(factor);
+  const float pow2 = __uint_as_float(bits & 0xff800000u);
+  const _Float16 m = (_Float16)__uint_as_float((bits & 0x007fffffu) | 0x3f800000u);
+  const half2_t mm = {m, m};
+  mhalf8_t r;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const half2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, false) * mm;
+    const half2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, true) * mm;
+    r[4 * i] = lo[0];
+    r[4 * i + 1] = lo[1];
+    r[4 * i + 2] = hi[0];
+    r[4 * i + 3] = hi[1];
+  }
+  return r;
+}
+
 template <int KV, int D, int W, int HPW>
 __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeParams p) {
   using G = Geo<KV, D, 1>;
@@ -125,7 +147,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   constexpr int WAVEB = decode_mfma_wave_bytes(HPW, D);
   uint8_t* my_lds = lds_raw + wave * WAVEB;            // this wave's tiles: per KV head K, then V
-  float* my_scales = reinterpret_cast<float*>(my_lds + HPW * TILEB);   // [2][TILE]: 1 / k_scale, 1 / v_scale per token
+  float* my_scales = reinterpret_cast<float*>(my_lds + HPW * TILEB);   // [TILE]: 1 / k_scale per token
   float (*red)[HPW * NHC * D] = reinterpret_cast<float (*)[HPW * NHC * D]>(lds_raw);   // [W][HPW * NHC * D], over the tiles
   float (*sm)[W] = reinterpret_cast<float (*)[W]>(lds_raw + W * WAVEB);                // [HPW * NHC][W]
   float (*sl)[W] = sm + HPW * NHC;                                                      // [HPW * NHC][W]
@@ -142,7 +164,10 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   const int kv_groups = p.num_kv_heads / HPW;
   int b, part, in;
   int members = 1;          // batch rows served at once: > 1 only for the shared partitions of a group
+  const int32_t* grows = nullptr;   // the group's rows when they are listed rather than consecutive
   if (p.group_desc) {
+    // Descriptors come from device memory: everything read from them is brought into range before
+    // it is used as an index, so that a corrupt descriptor gives wrong numbers, never a fault.
     int x = blockIdx.x;
     if (x < p.num_prefix_wgs) {
       in = x % p.inner;
@@ -150,14 +175,24 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       part = u % p.prefix_parts;
       const int32_t* desc = p.group_desc + 4 * (u / p.prefix_parts);
       if (part >= desc[2]) return;
-      b = desc[0];
-      members = desc[1];
+      members = min(desc[1], NHC / max(gq, 1));
+      if (members < 1) return;
+      if (p.group_rows) {
+        const int first = desc[0];
+        if (first < 0 || first + members > p.group_rows_len) return;
+        grows = p.group_rows + first;
+        b = grows[0];
+      } else {
+        b = desc[0];
+        members = min(members, p.batch - b);
+      }
+      if (b < 0 || b >= p.batch || members < 1) return;
     } else {
       x -= p.num_prefix_wgs;
       in = x % p.inner;
       const int u = x / p.inner;
       b = u / p.suffix_parts;
-      part = p.row_skip[b] + u % p.suffix_parts;
+      part = min(max(p.row_skip[b], 0), p.max_partitions) + u % p.suffix_parts;
       if (part >= p.max_partitions) return;
     }
   } else {
@@ -170,11 +205,14 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   const int sub = in / kv_groups;
   const int kvh0 = kvg * HPW;                        // first KV head of the workgroup
   // Columns of the matrix operand.  One row: query heads sub * 16 ... of the KV head.  A group's
-  // shared partition: column c = query head c % gq of row b + c / gq (gq * members <= 16).
+  // shared partition: column c = query head c % gq of the group's row c / gq (gq * members <= 16).
   const int cdiv = members > 1 ? gq : NHC + 1;
   const int nh = members > 1 ? members * gq : min(gq - sub * NHC, NHC);   // live columns per KV head
   auto first_head = [&](int hh) { return (kvh0 + hh) * gq + sub * NHC; };   // first query head behind KV head kvh0 + hh
-  auto col_row = [&](int c) { return b + c / cdiv; };
+  auto col_row = [&](int c) {
+    const int i = c / cdiv;
+    return grows ? min(max(grows[i], 0), p.batch - 1) : b + i;
+  };
   auto col_head = [&](int hh, int c) { return first_head(hh) + c % cdiv; };
 
   const int ctx = p.context_lens[b];
@@ -190,7 +228,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   int begin = 0, end = ctx;
   if (p.max_partitions > 1) {
     begin = part * p.partition_size;
-    end = (part == p.max_partitions - 1) ? ctx : min(begin + p.partition_size, ctx);
+    // the last partition takes whatever is left of the row's context; a shared one ends with the partition
+    end = (part == p.max_partitions - 1 && members == 1) ? ctx : min(begin + p.partition_size, ctx);
   }
   if (begin >= end) return;
 
@@ -300,6 +339,12 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     for (int r = 0; r < RL; ++r) {
       const int tk = token_of(r);
       const bool valid = !masked || (begin + tile * TILE + tk) < end;
+      // fp8: V is dequantised here, on its way into LDS (value = byte / v_scale, rounded to fp16), so
+      // that the probabilities stay pure numbers in [0, 256] when they are rounded to fp16 for the
+      // second product.  (Folding 1 / v_scale into the probability instead loses every key whose
+      // p / v_scale falls below fp16's smallest subnormal while its p still counts in the row sum.)
+      float inv_vs = 1.0f;
+      if constexpr (KV == KV_FP8) inv_vs = __builtin_amdgcn_rcpf(t.vs[r]);
 #pragma unroll
       for (int c = 0; c < G::NLD; ++c) {
 #pragma unroll
@@ -307,7 +352,9 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
           const int chunk = (c * 8 + j) * CPL + x;
           const int wpc = (KV == KV_FP8) ? 2 : 4;   // dwords per 8 source elements
           mhalf8_t kf = words_to_f16<KV>(&t.k[r][c * (G::LB / 4) + x * wpc]);
-          mhalf8_t vf = words_to_f16<KV>(&t.v[r][c * (G::LB / 4) + x * wpc]);
+          mhalf8_t vf;
+          if constexpr (KV == KV_FP8) vf = fp8_words_to_f16_scaled(&t.v[r][c * (G::LB / 4) + x * wpc], inv_vs);
+          else vf = words_to_f16<KV>(&t.v[r][c * (G::LB / 4) + x * wpc]);
           if (!valid) {
             // rows past the end: their scores are masked, and their V must not turn 0 * garbage into NaN
 #pragma unroll
@@ -320,20 +367,18 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       }
     }
     if constexpr (KV == KV_FP8) {
-      // 1 / scale per token, 0 for rows past the end (their V rows are zero, and 0 * 0 stays 0).  The 8
-      // lanes of a row group (and both heads' groups) hold the same values and write the same words.
+      // 1 / k_scale per token (applied to the scores after the first product), 0 for rows past the end
+      // (their scores are masked anyway).  The 8 lanes of a row group (and both heads' groups) hold the
+      // same values and write the same words.
 #pragma unroll
       for (int sb = 0; sb < NSUB; ++sb) {
-        float ik[4], iv[4];
+        float ik[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const bool valid = !masked || (begin + tile * TILE + token_of(4 * sb + r)) < end;
           ik[r] = valid ? __builtin_amdgcn_rcpf(t.ks[4 * sb + r]) : 0.0f;
-          iv[r] = valid ? __builtin_amdgcn_rcpf(t.vs[4 * sb + r]) : 0.0f;
         }
-        const int tok0 = token_of(4 * sb);
-        *(float4*)&my_scales[tok0] = make_float4(ik[0], ik[1], ik[2], ik[3]);
-        *(float4*)&my_scales[TILE + tok0] = make_float4(iv[0], iv[1], iv[2], iv[3]);
+        *(float4*)&my_scales[token_of(4 * sb)] = make_float4(ik[0], ik[1], ik[2], ik[3]);
       }
     }
   };
@@ -381,15 +426,13 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
         s2[hh][kb] = mfloat4_t{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
-    // fp8: 1 / scale of this lane's 8 keys (4kg .. 4kg+3 of both halves)
-    float iks[2][4], ivs[2][4];
+    // fp8: 1 / k_scale of this lane's 8 keys (4kg .. 4kg+3 of both halves)
+    float iks[2][4];
     if constexpr (KV == KV_FP8) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         const float4 a = *(const float4*)&my_scales[16 * kb + 4 * kg];
-        const float4 b2 = *(const float4*)&my_scales[TILE + 16 * kb + 4 * kg];
         iks[kb][0] = a.x; iks[kb][1] = a.y; iks[kb][2] = a.z; iks[kb][3] = a.w;
-        ivs[kb][0] = b2.x; ivs[kb][1] = b2.y; ivs[kb][2] = b2.z; ivs[kb][3] = b2.w;
       }
     }
 #pragma unroll
@@ -456,18 +499,11 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
-          if constexpr (KV == KV_FP8) {
-            // the row sum takes the probability, the product the probability / v_scale
-            const float p0 = __builtin_amdgcn_exp2f(s[hh][kb][e]), p1 = __builtin_amdgcn_exp2f(s[hh][kb][e + 1]);
-            psum += p0 + p1;
-            pb[hh][4 * kb + e] = (_Float16)(p0 * ivs[kb][e]);
-            pb[hh][4 * kb + e + 1] = (_Float16)(p1 * ivs[kb][e + 1]);
-          } else {
-            const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
-            psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
-            pb[hh][4 * kb + e] = h[0];
-            pb[hh][4 * kb + e + 1] = h[1];
-          }
+          // the row sum adds exactly the fp16 values that the second product multiplies
+          const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
+          psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
+          pb[hh][4 * kb + e] = h[0];
+          pb[hh][4 * kb + e + 1] = h[1];
         }
       l_run[hh] += psum;
     }

@@ -9,8 +9,10 @@
 // nominal one.  pa_hbm_read_probe streams a buffer once with 16-byte loads (ordinary or non-temporal),
 // every workgroup its own contiguous chunk, four loads per lane in flight: the plain read rate of the
 // GPU, which the decode kernels' achieved bytes per second are put beside.  No counterparts in the reference.
+// Part of the measuring library libpa_probes.so (pa_probes.h), not of the product library.
 #include "pa_common.hpp"
 #include "pa_host.hpp"
+#include "pa_probes.h"
 
 namespace pa {
 
@@ -77,8 +79,9 @@ __global__ __launch_bounds__(256) void hbm_read_probe_kernel(const uint8_t* __re
 using namespace pa;
 
 extern "C" int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, int streaming, uint32_t* sink,
-                                     void* stream) {
+                                     int64_t sink_words, void* stream) {
   if (!src || !sink) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: null pointer");
+  if (sink_words < groups) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: sink must hold one word per workgroup");
   if (groups <= 0 || groups > 0x7fffffff || bytes <= 0) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: bad size");
   if (!aligned16(src)) return fail(PA_ERR_BAD_ARG, "pa_hbm_read_probe: buffer must be 16-byte aligned");
   const int64_t per_group = bytes / 16 / groups;
@@ -94,14 +97,17 @@ extern "C" int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t gro
   return per_group * groups * 16;   // bytes read
 }
 
-extern "C" int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t steps, float* sink, void* stream) {
+extern "C" int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t num_operands, int64_t steps, float* sink,
+                                      int64_t sink_floats, void* stream) {
   if (!operands_f16 || !sink) return fail(PA_ERR_BAD_ARG, "pa_mfma_rate_probe: null pointer");
   if (steps <= 0 || steps > (int64_t(1) << 24)) return fail(PA_ERR_BAD_ARG, "pa_mfma_rate_probe: steps must be in 1 .. 2^24");
+  if (num_operands < kProbeOperands) return fail(PA_ERR_BAD_ARG, "pa_mfma_rate_probe: operands_f16 must hold 65536 values");
   int dev = 0;
   hipDeviceProp_t prop;
   if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
     return fail(PA_ERR_LAUNCH, "pa_mfma_rate_probe: cannot query the device");
   const int cus = prop.multiProcessorCount;
+  if (sink_floats < cus) return fail(PA_ERR_BAD_ARG, "pa_mfma_rate_probe: sink must hold one float per compute unit");
   hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned)cus), dim3(512), 0, (hipStream_t)stream,
                      (const _Float16*)operands_f16, steps, sink);
   const int rc = check_launch("pa_mfma_rate_probe");

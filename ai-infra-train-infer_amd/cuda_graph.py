@@ -15,8 +15,8 @@ row.  Here a buffer is created with, and before every replay reset to, its paddi
 `slot_mapping` -1 (the writers skip it), everything else 0 (`context_lens` 0: the row reads
 nothing and its output is zero).  Other names take a value through `buffer_fill={name: value}`.
 
-The recorded region must not allocate: every kernel of this library takes its workspace from a
-per-stream buffer that the warm-up runs (outside the recording) have already sized.
+The recorded region must not allocate: the partitioned decode launches take their partials from
+the device's workspace for graphs, which the warm-up runs (outside the recording) have sized.
 """
 from typing import Callable, Dict, List, Optional, Tuple
 
@@ -58,9 +58,11 @@ class CUDAGraphRunner:
         for name, shape in extra_buffer_shapes.items():
             buffers[name] = torch.full(tuple(shape), fill.get(name, 0), dtype=torch.int32, device=device)
         extra = {name: buffers[name] for name in extra_buffer_shapes}
+        from .attention import sizing_graph_workspace
         with torch.inference_mode():
-            for _ in range(max(1, num_warmup)):         # sizes workspaces and library handles
-                model_forward_fn(buffers["input_ids"], buffers["positions"], **extra)
+            with sizing_graph_workspace():
+                for _ in range(max(1, num_warmup)):     # sizes the graphs' workspace and library handles
+                    model_forward_fn(buffers["input_ids"], buffers["positions"], **extra)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):

@@ -50,9 +50,12 @@ class ModelRunnerConfig:
     device: str = "cuda"
     enable_cuda_graph: bool = True
     max_cuda_graph_batch_size: int = 64
-    # decode steps look for rows that share prefixes as the same blocks (n samples of a prompt,
-    # forks of a cached prefix) and read a shared partition once per group; eager steps only
-    share_prefix_decode: bool = False
+    # decode steps read a prefix that several rows share as the same blocks (n samples of a prompt,
+    # forks of a cached prefix) once per group of rows instead of once per row.  The groups are kept
+    # where the rows are: DecodeState updates them when a row is admitted or retired, prepare_decode
+    # keeps the last step's groups for as long as the batch's first blocks stay what they were.
+    share_prefix_decode: bool = True
+    prefix_partition_sizes: Tuple[int, ...] = (1024, 512)     # tokens; coarsest first
 
 
 def slots_for_range(block_table, start, end, block_size):
@@ -76,7 +79,12 @@ class DecodeState:
     """
 
     def __init__(self, max_batch: int, max_blocks_per_seq: int, block_size: int, num_blocks: int,
-                 device: str = "cuda"):
+                 device: str = "cuda", num_q_heads: Optional[int] = None, num_kv_heads: Optional[int] = None,
+                 prefix_partition_sizes: Tuple[int, ...] = (1024, 512)):
+        """num_q_heads / num_kv_heads: give them and the state also keeps the groups of rows that share
+        a prefix as the same physical blocks (rebuilt when a row is admitted or retired, never per
+        step), as device descriptors for pa_decode_shared_prefix; prefix_partition_sizes are the
+        partition sizes such a launch may use, coarsest first."""
         dev = torch.device(device)
         self.max_batch, self.max_blocks = int(max_batch), int(max_blocks_per_seq)
         self.block_size, self.num_blocks = int(block_size), int(num_blocks)
@@ -93,6 +101,23 @@ class DecodeState:
         self._fresh_rows = set()                        # host copy of the same
         self._lens = [0] * max_batch                    # tokens in the cache, per row (0 = free)
         self._tables = [[] for _ in range(max_batch)]   # block ids, per row
+        # ---- rows that share prefixes ---------------------------------------------------------------
+        self._heads = (int(num_q_heads), int(num_kv_heads)) if num_q_heads and num_kv_heads else None
+        self.max_group_rows = 16 // max(1, self._heads[0] // self._heads[1]) if self._heads else 0
+        self.prefix_partition_sizes = tuple(sorted(
+            (int(x) for x in prefix_partition_sizes if int(x) > 0 and int(x) % self.block_size == 0 and int(x) % 16 == 0
+             and int(x) <= self.max_blocks * self.block_size), reverse=True))
+        self.tracks_prefixes = self.max_group_rows >= 2 and bool(self.prefix_partition_sizes) and max_batch >= 2
+        self.max_groups = max_batch // 2
+        self.prefix_partition_size: Optional[int] = None    # of the groups now on the device; None: no groups
+        self.prefix_groups_host: List[Tuple[List[int], int]] = []
+        self._groups_dirty = False
+        if self.tracks_prefixes:
+            # one buffer, so that an update is one copy: group_desc [G, 4] | group_rows [B] | row_skip [B]
+            self._groups_dev = torch.zeros(4 * self.max_groups + 2 * max_batch, dtype=torch.int32, device=dev)
+            self._group_desc = self._groups_dev[:4 * self.max_groups].view(-1, 4)
+            self._group_rows = self._groups_dev[4 * self.max_groups:4 * self.max_groups + max_batch]
+            self._row_skip = self._groups_dev[4 * self.max_groups + max_batch:]
 
     @property
     def rows_in_use(self) -> int:
@@ -128,6 +153,7 @@ class DecodeState:
         self._fresh_rows.add(row)
         self._lens[row] = int(num_cached_tokens)
         self._tables[row] = list(block_table)
+        self._groups_dirty = self.tracks_prefixes
         return row
 
     def retire(self, row: int) -> List[int]:
@@ -135,7 +161,72 @@ class DecodeState:
         self.context_lens[row].fill_(0)
         self._fresh_rows.discard(row)
         blocks, self._tables[row], self._lens[row] = self._tables[row], [], 0
+        self._groups_dirty = self.tracks_prefixes
         return blocks
+
+    # ---- rows that share prefixes ---------------------------------------------------------------------
+    # Full blocks never change while one of their owners lives, so what a set of rows shares is fixed
+    # from the moment the last of them is admitted until the first of them retires: the groups are
+    # rebuilt on those two events only, on the host, from the block-id lists the state already keeps
+    # (rows that share anything share their first block: one dictionary pass finds the candidates),
+    # and shipped to the device in one small copy.  A step costs nothing.
+
+    def sync_prefix_groups(self):
+        """Bring the device descriptors up to date with the rows admitted and retired since the last
+        call.  Called by step() and set_context(); a launch over descriptors that still name a retired
+        row would skip that row's group."""
+        if not self._groups_dirty:
+            return
+        from .attention import choose_prefix_partition, find_prefix_groups_anywhere
+        self._groups_dirty = False
+        active = self.active_rows()
+        tables = [self._tables[r] for r in active]
+        lens = [self._lens[r] for r in active]
+        hq, hkv = self._heads
+
+        def find(size):
+            return find_prefix_groups_anywhere(tables, lens, self.block_size, hq, hkv, size, rows=active)
+
+        size, groups = choose_prefix_partition(find, self.prefix_partition_sizes)
+        groups = groups[:self.max_groups]
+        had = self.prefix_partition_size is not None
+        self.prefix_partition_size, self.prefix_groups_host = (size, groups) if groups else (None, [])
+        if not groups and not had:
+            return                                     # nothing on the device names a row
+        host = torch.zeros(self._groups_dev.numel(), dtype=torch.int32)
+        desc = host[:4 * self.max_groups].view(-1, 4)
+        rows_flat = host[4 * self.max_groups:4 * self.max_groups + self.max_batch]
+        skip = host[4 * self.max_groups + self.max_batch:]
+        cursor = 0
+        for i, (members, tokens) in enumerate(groups):
+            parts = tokens // size
+            desc[i, 0], desc[i, 1], desc[i, 2] = cursor, len(members), parts
+            for r in members:
+                rows_flat[cursor] = r
+                skip[r] = parts
+                cursor += 1
+        self._groups_dev.copy_(host.pin_memory(), non_blocking=True)
+
+    def prefix_groups(self, batch: int, partition_size: Optional[int] = None, for_graph: bool = False):
+        """PrefixGroups over the state's device descriptors for the first `batch` rows, or None when
+        no rows share a prefix.  for_graph: the descriptors at their full capacity whatever they hold
+        now (empty groups cost a workgroup that returns at once), for partition_size - what a
+        recorded launch must be sized with."""
+        from .attention import PrefixGroups
+        if not self.tracks_prefixes:
+            return None
+        if for_graph:
+            size = int(partition_size)
+            parts = -(-self.max_blocks * self.block_size // size)
+            return PrefixGroups(size, self._group_desc, self._group_rows, self._row_skip[:batch], self.max_groups,
+                                self.max_group_rows, parts, 0)
+        self.sync_prefix_groups()
+        if self.prefix_partition_size is None:
+            return None
+        size = self.prefix_partition_size
+        groups = self.prefix_groups_host
+        return PrefixGroups(size, self._group_desc, self._group_rows, self._row_skip[:batch], len(groups),
+                            max(len(m) for m, _ in groups), max(t for _, t in groups) // size, 0, groups=groups)
 
     def rows_needing_block(self) -> List[int]:
         """Active rows whose next token opens a block they do not have yet."""
@@ -151,6 +242,7 @@ class DecodeState:
         since that step keep the token they were admitted with."""
         from . import _native
         lib = _native.load()
+        self.sync_prefix_groups()
         n = self.rows_in_use
         if next_tokens is not None:
             next_tokens = next_tokens.reshape(-1)
@@ -200,11 +292,20 @@ class DecodeState:
                 self._lens[r] += 1
         self._fresh_rows.clear()
 
-    def set_context(self, batch: Optional[int] = None):
-        """Point the attention layers at the first `batch` rows (default: the rows in use)."""
+    def set_context(self, batch: Optional[int] = None, share_prefixes: bool = True,
+                    graph_partition_size: Optional[int] = None):
+        """Point the attention layers at the first `batch` rows (default: the rows in use).
+        share_prefixes: hand them the groups of rows that share a prefix, when there are any;
+        graph_partition_size: the descriptors at full capacity for that partition size instead (what
+        a graph is recorded over)."""
         n = self.rows_in_use if batch is None else batch
+        groups = None
+        if graph_partition_size is not None:
+            groups = self.prefix_groups(n, graph_partition_size, for_graph=True)
+        elif share_prefixes:
+            groups = self.prefix_groups(n)
         set_context(False, slot_mapping=self.slot_mapping[:n], context_lens=self.context_lens[:n],
-                    block_tables=self.block_tables[:n])
+                    block_tables=self.block_tables[:n], prefix_groups=groups)
         return n
 
 
@@ -224,8 +325,12 @@ class ModelRunner:
         self._graph_pool = None
         self._graph_vars: Optional[Dict[str, torch.Tensor]] = None
         self._graph_batch_sizes: List[int] = []
-        self._state_graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._state_graphs: Dict[Tuple[int, int, Optional[int]], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._hf_model: Optional[torch.nn.Module] = None
+        self._prefix_groups_kept = None          # (signature of the batch, PrefixGroups or None) of the last decode step
+        # how run_decode_state ran its steps: replays of a graph recorded over the shared-prefix launch,
+        # replays of a plain graph, eager forwards
+        self.decode_state_stats = {"shared_prefix_graph": 0, "plain_graph": 0, "eager": 0}
 
     # ---------------------------------------------------------------- cache binding
 
@@ -328,9 +433,7 @@ class ModelRunner:
             lens[i] = len(toks)
         groups = None
         if getattr(self.config, "share_prefix_decode", False) and self._device() != "cpu":
-            from .attention import prepare_prefix_groups
-            groups = prepare_prefix_groups([seq["block_table"] for seq in sequences], lens.tolist(), self.block_size,
-                                           self.config.num_heads, self.config.num_kv_heads, self._device())
+            groups = self._decode_prefix_groups([seq["block_table"] for seq in sequences], lens.tolist())
         set_context(
             is_prefill=False,
             slot_mapping=self._to_device(slots, torch.int32),
@@ -339,6 +442,43 @@ class ModelRunner:
             prefix_groups=groups,
         )
         return self._to_device(ids, torch.long), self._to_device(pos, torch.long)
+
+    def _decode_prefix_groups(self, tables, lens):
+        """Groups of rows that share a prefix, for prepare_decode.  Finding them walks block-id lists,
+        so the last result is kept and reused while it provably still holds: same batch size, same
+        first block in every row (rows that share anything share their first block, so new sharing
+        cannot appear without one of these changing), and every member of every group still has its
+        group's last shared block where it was and a context that covers the shared tokens (shared
+        blocks are full blocks, which never change while an owner lives).  A step with an unchanged
+        batch costs one pass over the rows."""
+        cfg = self.config
+        if 16 // max(1, cfg.num_heads // cfg.num_kv_heads) < 2:
+            return None
+        key = (len(tables),) + tuple(t[0] if len(t) else -1 for t in tables)
+        kept = self._prefix_groups_kept
+        if kept is not None and kept[0] == key:
+            pg = kept[1]
+            if pg is None:
+                return None
+            bs = self.block_size
+            for members, tokens in pg.groups:
+                last = tokens // bs - 1
+                lead = tables[members[0]]
+                if any(len(tables[r]) <= last or tables[r][last] != lead[last] or lens[r] < tokens for r in members):
+                    break
+            else:
+                return pg
+        sizes = [x for x in cfg.prefix_partition_sizes if x % self.block_size == 0 and x % 16 == 0]
+        pg = None
+        if sizes:
+            from .attention import choose_prefix_partition, find_prefix_groups_anywhere, shared_prefix_descriptors
+            size, groups = choose_prefix_partition(
+                lambda x: find_prefix_groups_anywhere(tables, lens, self.block_size, cfg.num_heads, cfg.num_kv_heads, x),
+                sizes)
+            if groups:
+                pg = shared_prefix_descriptors(groups, len(tables), self._device(), size)
+        self._prefix_groups_kept = (key, pg)
+        return pg
 
     # ---------------------------------------------------------------- forward
 
@@ -507,6 +647,7 @@ class ModelRunner:
         if batch_sizes is None:
             max_bs = min(self.config.max_cuda_graph_batch_size, 64)
             batch_sizes = [1, 2, 4, 8] + list(range(16, max_bs + 1, 16))
+        from .attention import sizing_graph_workspace
         self._graph_batch_sizes = sorted(batch_sizes)
         max_bs = max(batch_sizes)
         dev = self.config.device
@@ -523,7 +664,8 @@ class ModelRunner:
             set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
                         block_tables=gv["block_tables"][:bs])
             # warm-up outside the capture: library handles, allocator warm-up
-            self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
+            with sizing_graph_workspace():
+                self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
             torch.cuda.synchronize()
             with torch.cuda.graph(graph, pool=self._graph_pool):
                 out = self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
@@ -542,7 +684,7 @@ class ModelRunner:
         from .attention import decode_workspace_bytes, reserve_decode_workspace
         cfg = self.config
         reserve_decode_workspace(torch.device(cfg.device),
-                                 decode_workspace_bytes(max_batch, cfg.num_heads, cfg.head_dim))
+                                 decode_workspace_bytes(max_batch, cfg.num_heads, cfg.head_dim), for_graphs=True)
 
     def _run_with_cuda_graph(self, input_ids, positions):
         bs = input_ids.size(0)
@@ -570,25 +712,37 @@ class ModelRunner:
     @torch.inference_mode()
     def capture_decode_state_graphs(self, state: DecodeState, batch_sizes: Optional[List[int]] = None):
         """Record the decode forward over the first n rows of `state` for each n: the graph's
-        inputs are the state's own tensors, so a replay needs no copies at all."""
+        inputs are the state's own tensors, so a replay needs no copies at all.  When the state keeps
+        groups of rows that share a prefix (and config.share_prefix_decode), a second graph per n and
+        partition size is recorded over its group descriptors - at their full capacity, empty groups
+        included, since a recorded launch cannot be resized - and run_decode_state replays that one
+        whenever the state holds a group."""
+        from .attention import sizing_graph_workspace
         if not torch.cuda.is_available() or self.model is None:
             return
         if batch_sizes is None:
             batch_sizes = sorted({b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < state.max_batch}
                                  | {state.max_batch})
         self._reserve_decode_workspace(max(batch_sizes))
+        variants = [None]
+        if state.tracks_prefixes and getattr(self.config, "share_prefix_decode", False):
+            variants += list(state.prefix_partition_sizes)
         for bs in sorted(batch_sizes, reverse=True):
-            state.set_context(bs)
-            self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                out = self.model(state.input_ids[:bs], positions=state.positions[:bs])
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
-            self._state_graphs[(id(state), bs)] = (graph, out)
-            torch.cuda.synchronize()
-            reset_context()
+            for psize in variants:
+                if psize is not None and bs < 2:
+                    continue
+                state.set_context(bs, share_prefixes=False, graph_partition_size=psize)
+                with sizing_graph_workspace():
+                    self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    out = self.model(state.input_ids[:bs], positions=state.positions[:bs])
+                if self._graph_pool is None:
+                    self._graph_pool = graph.pool()
+                self._state_graphs[(id(state), bs, psize)] = (graph, out)
+                torch.cuda.synchronize()
+                reset_context()
 
     @torch.inference_mode()
     def run_decode_state(self, state: DecodeState) -> torch.Tensor:
@@ -596,13 +750,19 @@ class ModelRunner:
         if self.model is None:
             raise RuntimeError("ModelRunner.run_decode_state: no model bound")
         n = state.rows_in_use
+        share = getattr(self.config, "share_prefix_decode", False)
+        state.sync_prefix_groups()
         if self.config.enable_cuda_graph:
-            sizes = sorted(bs for (sid, bs) in self._state_graphs if sid == id(state) and bs >= n)
-            if sizes:
-                graph, out = self._state_graphs[(id(state), sizes[0])]
-                graph.replay()
-                return out[:n]
-        state.set_context(n)
+            psize = state.prefix_partition_size if share else None
+            for want in ((psize, None) if psize is not None else (None,)):
+                sizes = sorted(bs for (sid, bs, ps) in self._state_graphs if sid == id(state) and ps == want and bs >= n)
+                if sizes:
+                    graph, out = self._state_graphs[(id(state), sizes[0], want)]
+                    graph.replay()
+                    self.decode_state_stats["plain_graph" if want is None else "shared_prefix_graph"] += 1
+                    return out[:n]
+        self.decode_state_stats["eager"] += 1
+        state.set_context(n, share_prefixes=share)
         logits = self.model(state.input_ids[:n], positions=state.positions[:n])
         reset_context()
         return logits
@@ -610,6 +770,7 @@ class ModelRunner:
     def invalidate_cuda_graphs(self):
         """Drop every recorded graph (after a weight update)."""
         self._state_graphs.clear()
+        self._prefix_groups_kept = None
         self._graphs.clear()
         self._graph_outputs.clear()
         self._graph_pool = None

@@ -32,6 +32,31 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+_PROBES = None
+
+
+def load_probes():
+    """The measuring library (ai-infra-train-infer_amd/csrc/probes/libpa_probes.so, pa_probes.h): the
+    decode launch with loads only, the plain HBM read rate, the sustained matrix-pipe rate.  Built by
+    the package's build step beside the product library; the product never loads it."""
+    global _PROBES
+    if _PROBES is None:
+        import ctypes
+        import torch  # noqa: F401  (its HIP runtime first, as for the product library)
+        path = os.path.join(ROOT, "ai-infra-train-infer_amd", "csrc", "probes", "libpa_probes.so")
+        if not os.path.exists(path):
+            raise RuntimeError("libpa_probes.so is not built (%s): run `python ai-infra-train-infer_amd/build.py`" % path)
+        lib = ctypes.CDLL(path)
+        i64, i32, ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+        lib.pa_probes_last_error.restype, lib.pa_probes_last_error.argtypes = ctypes.c_char_p, []
+        lib.pa_decode_load_probe.restype = i32
+        lib.pa_decode_load_probe.argtypes = [ptr, i32, i64, ptr, ptr, ptr, ptr, i32, ptr, i64, i64, ptr, i64, i64, i64, i64,
+                                             i64, i64, i64, i64, ptr, i64, i32, i32, i32, ptr]
+        lib.pa_mfma_rate_probe.restype, lib.pa_mfma_rate_probe.argtypes = i64, [ptr, i64, i64, ptr, i64, ptr]
+        lib.pa_hbm_read_probe.restype, lib.pa_hbm_read_probe.argtypes = i64, [ptr, i64, i64, i32, ptr, i64, ptr]
+        _PROBES = lib
+    return _PROBES
+
 
 def algorithmic_bytes(batch, ctx, hq, hkv, d, bs, fp8):
     """K and V of every context token once, fp8 scales, q in and out, table entries and lens."""
@@ -261,13 +286,13 @@ def other_decode_configs(pa, torch, dev, launches):
     # the same batch with the samples of a prompt named as a group: partitions inside the shared prefix are
     # read once per prompt (what ModelRunnerConfig.share_prefix_decode does from the host's block-id lists)
     host_tables = [row[:(n + BS - 1) // BS] for row, n in zip(w4["block_tables"].cpu().tolist(), lens4)]
-    pg4 = pa.prepare_prefix_groups(host_tables, lens4, BS, HQ, HKV, dev)
-    assert pg4 is not None and pg4["groups"] == [(8 * i, 8, 1024) for i in range(32)], pg4 and pg4["groups"]
+    pg4 = pa.prepare_prefix_groups(host_tables, lens4, BS, HQ, HKV, dev, anywhere=True)
+    assert pg4 is not None and pg4.groups == [(list(range(8 * i, 8 * i + 8)), 1024) for i in range(32)], pg4 and pg4.groups
     fns["cfg4_shared_prefix"] = lambda: pa.paged_decode_shared_prefix(
-        w4["q"], w4["k_cache"], w4["v_cache"], w4["block_tables"], w4["context_lens"], scale, pg4["groups"],
-        partition_size=pg4["partition_size"], out=w4["out"], descriptors=pg4["descriptors"])
+        w4["q"], w4["k_cache"], w4["v_cache"], w4["block_tables"], w4["context_lens"], scale, None,
+        out=w4["out"], descriptors=pg4)
     meta["cfg4_shared_prefix"] = dict(workload=meta["cfg4"]["workload"] + "; shared partitions (%d tokens, the group finder's "
-                                      "choice) read once per prompt, matrix kernel + merge" % pg4["partition_size"],
+                                      "choice) read once per prompt, matrix kernel + merge" % pg4.partition_size,
                                       kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
     t = time_alternating(torch, fns, launches)
@@ -394,7 +419,7 @@ def hbm_stream_read(pa, torch, dev, launches):
     """The plain read rate of the GPU: pa_hbm_read_probe over a 1 GiB buffer (every workgroup streams
     its own contiguous share once, 16-byte loads), for four workgroup counts, alternated, medians.
     1 GiB exceeds the 256 MB of last-level cache, so every launch reads HBM."""
-    lib = pa._native.load()
+    lib = load_probes()
     nbytes = 1 << 30
     buf = torch.ones(nbytes // 4, dtype=torch.float32, device=dev)
     sink = torch.empty(1 << 15, dtype=torch.int32, device=dev)
@@ -406,8 +431,8 @@ def hbm_stream_read(pa, torch, dev, launches):
             groups = cus * mult
 
             def fn(groups=groups, streaming=streaming):
-                got = lib.pa_hbm_read_probe(buf.data_ptr(), nbytes, groups, streaming, sink.data_ptr(), stream)
-                assert got == nbytes, lib.pa_last_error()
+                got = lib.pa_hbm_read_probe(buf.data_ptr(), nbytes, groups, streaming, sink.data_ptr(), sink.numel(), stream)
+                assert got == nbytes, lib.pa_probes_last_error()
 
             fns["%sworkgroups_%d" % ("" if streaming else "ordinary_loads_", groups)] = fn
     t = time_alternating(torch, fns, max(20, launches // 5), warmup=3)
@@ -429,7 +454,7 @@ def mfma_ceiling(pa, torch, dev):
     v_mfma_f32_32x32x16_f16 on every SIMD, operands from registers, launches of ~10 ms) on constant
     operands and on N(0,1) operands, alternated, median of 5.  The clocks drop under the matrix
     pipe, further when the operands toggle, so the nominal dense-fp16 peak is not a sustained rate."""
-    lib = pa._native.load()
+    lib = load_probes()
     g = torch.Generator(device=dev).manual_seed(14)
     ops = {"constant_operands": torch.ones(65536, dtype=torch.float16, device=dev),
            "normal_operands": torch.randn(65536, generator=g, device=dev, dtype=torch.float32).half()}
@@ -442,10 +467,10 @@ def mfma_ceiling(pa, torch, dev):
         for name, t in ops.items():
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
-            flops = lib.pa_mfma_rate_probe(t.data_ptr(), steps, sink.data_ptr(), stream)
+            flops = lib.pa_mfma_rate_probe(t.data_ptr(), t.numel(), steps, sink.data_ptr(), sink.numel(), stream)
             stop.record()
             torch.cuda.synchronize()
-            assert flops > 0, lib.pa_last_error()
+            assert flops > 0, lib.pa_probes_last_error()
             if rep_:
                 res[name].append(start.elapsed_time(stop))
     out = {"what": "pa_mfma_rate_probe: nothing but independent v_mfma_f32_32x32x16_f16 on every SIMD, "
@@ -796,14 +821,14 @@ def main():
         w["probe_ws"] = torch.empty(max(pbytes, 256), dtype=torch.uint8, device=dev)
 
         def probe(w=w, fp8=fp8, psize=psize, parts=parts, hpw=hpw):
-            rc = lib.pa_decode_load_probe(
+            rc = load_probes().pa_decode_load_probe(
                 w["q"].data_ptr(), 0, HQ * D, w["k_cache"].data_ptr(), w["v_cache"].data_ptr(),
                 w["k_scale"].data_ptr() if fp8 else None, w["v_scale"].data_ptr() if fp8 else None,
                 pa._native.DTYPE_FP8_E4M3 if fp8 else pa._native.DTYPE_F16, w["block_tables"].data_ptr(),
                 w["block_tables"].stride(0), w["block_tables"].shape[1], w["context_lens"].data_ptr(),
                 B, HQ, HKV, D, BS, w["num_blocks"], max(psize, 16), parts, w["probe_ws"].data_ptr(),
                 w["probe_ws"].numel(), 0, hpw, 0, stream)
-            assert rc == 0, lib.pa_last_error()
+            assert rc == 0, load_probes().pa_probes_last_error()
 
         if "probe" in sections:
             fns[kind + "_probe"] = probe

@@ -44,7 +44,7 @@ extern "C" {
 #define PA_DTYPE_F32 2
 #define PA_DTYPE_FP8_E4M3 3 /* OCP e4m3fn, the layout of torch.float8_e4m3fn */
 
-/* Library ABI version (bumped when a signature changes); 2 = launch shape as per-call arguments. */
+/* Library ABI version (bumped when a signature changes); 3 = listed group rows in pa_decode_shared_prefix. */
 int pa_version(void);
 
 /* Message for the last non-zero return code on this thread ("" if none). */
@@ -204,17 +204,22 @@ int pa_decode_partials(const void* q, int q_dtype, int64_t q_token_stride, const
  * reference reads a shared block once per sequence that maps it (blocks carry a ref_count for
  * prefix sharing, src/inference/kv_cache.py:42-62, 190-210).
  * Arguments as pa_decode (partition_size > 0; the matrix kernel, one KV head per wave), plus:
- *   group_desc            device int32 [num_groups][4]: first batch row, number of rows (consecutive),
- *                         shared partitions, unused.  The first shared_partitions x partition_size
- *                         tokens of every row of a group must map to the same physical blocks as
- *                         the group's first row, and every row's context must hold them.
+ *   group_desc            device int32 [num_groups][4]: first, number of rows, shared partitions,
+ *                         unused.  The first shared_partitions x partition_size tokens of every row
+ *                         of a group must map to the same physical blocks as the group's first row,
+ *                         and every row's context must hold them.  A group of 0 shared partitions
+ *                         is empty (padding: a recorded HIP graph keeps num_groups fixed).
+ *   group_rows            NULL: a group's rows are the consecutive batch rows first .. first + rows - 1.
+ *                         Else device int32 [num_group_rows]: the group's rows are
+ *                         group_rows[first .. first + rows - 1], any batch rows in any order.
  *   max_group_rows        most rows of any group; rows x (num_q_heads / num_kv_heads) <= 16
  *   max_shared_partitions most shared partitions of any group
  *   row_skip              device int32 [batch]: the row's group's shared partitions, 0 for rows of
  *                         no group
  *   max_own_partitions    most partitions any row computes itself:
  *                         >= ceil(context_len / partition_size) - row_skip[row] for every row
- * The launch trusts the descriptors (pa_check_shared_prefix counts what is wrong with them).
+ * The launch trusts what the descriptors say is shared (pa_check_shared_prefix counts what is wrong
+ * with them); indices read from them are clamped, so that a corrupt descriptor cannot fault.
  */
 int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
                             const void* v_cache, const float* k_scale, const float* v_scale,
@@ -225,6 +230,7 @@ int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_token_stride, 
                             int64_t num_blocks, float scale, int64_t partition_size,
                             int64_t max_partitions, void* workspace, int64_t workspace_bytes,
                             int waves_per_workgroup, const int32_t* group_desc, int64_t num_groups,
+                            const int32_t* group_rows, int64_t num_group_rows,
                             int64_t max_group_rows, int64_t max_shared_partitions,
                             const int32_t* row_skip, int64_t max_own_partitions, void* stream);
 
@@ -241,47 +247,8 @@ int pa_decode_shared_prefix(const void* q, int q_dtype, int64_t q_token_stride, 
 int pa_check_shared_prefix(const int32_t* block_tables, int64_t bt_stride, int64_t table_width,
                            const int32_t* context_lens, int64_t batch, int64_t block_size,
                            int64_t partition_size, const int32_t* group_desc, int64_t num_groups,
+                           const int32_t* group_rows, int64_t num_group_rows,
                            const int32_t* row_skip, int32_t* counts, void* stream);
-
-/*
- * Timing aid: the launch of pa_decode_partials with the attention arithmetic taken out.  Every
- * K, V, scale and table load of the real launch is issued from the same lanes in the same order
- * and every loaded word is consumed (a checksum lands in `workspace`), but no dot product,
- * exponential or accumulation is done.  Its duration is what the memory system needs for this
- * access pattern alone - the ceiling the decode kernel is measured against besides the nominal
- * HBM rate.  Arguments as pa_decode_partials (no scale factor); the workspace contents are
- * meaningless afterwards.  No counterpart in the reference.
- */
-int pa_decode_load_probe(const void* q, int q_dtype, int64_t q_token_stride, const void* k_cache,
-                         const void* v_cache, const float* k_scale, const float* v_scale,
-                         int kv_dtype, const int32_t* block_tables, int64_t bt_stride,
-                         int64_t table_width, const int32_t* context_lens, int64_t batch,
-                         int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
-                         int64_t block_size, int64_t num_blocks, int64_t partition_size,
-                         int64_t max_partitions, void* workspace, int64_t workspace_bytes,
-                         int waves_per_workgroup, int kv_heads_per_wave, int q_heads_per_wave,
-                         void* stream);
-
-/*
- * Measuring aid: the rate the matrix pipe sustains.  Runs nothing but independent
- * v_mfma_f32_32x32x16_f16 on every SIMD (one workgroup of 8 waves per compute unit, `steps` x 16
- * products per wave) on operands taken from `operands_f16` (65536 fp16 values: constants, or the
- * kind of data the attention kernels see - the clocks of the part depend on how the operands
- * toggle).  `sink` receives one float per compute unit (at least 1024 floats).  Returns the number
- * of floating-point operations of the launch (time it with events on `stream`), or a negative
- * error code.  No counterpart in the reference.
- */
-int64_t pa_mfma_rate_probe(const void* operands_f16, int64_t steps, float* sink, void* stream);
-
-/*
- * Measuring aid: the plain read rate of the GPU.  `groups` workgroups of 256 threads each stream
- * their own contiguous share of `bytes` bytes at `src` once (16-byte loads, four per lane in flight;
- * streaming != 0: non-temporal loads, the way the decode kernels read private K and V)
- * and leave the XOR of their words, folded to 32 bits, in sink[group].  Returns the number of bytes
- * read (bytes rounded down to 16 x groups), or a negative error code.  No counterpart in the reference.
- */
-int64_t pa_hbm_read_probe(const void* src, int64_t bytes, int64_t groups, int streaming, uint32_t* sink,
-                          void* stream);
 
 /*
  * Merge reduction over partitions.

@@ -134,9 +134,9 @@ def config3(seed=1003, batch=4, lo=16384, hi=32768):
     return make_case(seed, lens, blocks)
 
 
-def config4(seed=1004, prompts=32, samples=8, prefix=1024, lo=64, hi=512):
+def config4(seed=1004, prompts=32, samples=8, prefix=1024, lo=64, hi=512, cache="fp16"):
     """32 prompts x 8 samples sharing a 1024-token prefix (aliased physical blocks)."""
     suffix = uniform_lens(seed, prompts * samples, lo, hi)
     lens = [prefix + s for s in suffix]
     own = sum((l + 15) // 16 - (prefix // 16 if i % samples else 0) for i, l in enumerate(lens))
-    return make_case(seed, lens, own + 64, shared_prefix=(samples, prefix // 16))
+    return make_case(seed, lens, own + 64, shared_prefix=(samples, prefix // 16), cache=cache)

@@ -318,10 +318,10 @@ def test_table_check_counts_what_the_kernels_would_clamp(pa, gpu, monkeypatch):
     check(got.cpu(), oracle_decode(c), "fp16")
 
 
-def test_workspace_is_per_device_grows_outside_captures_and_outlives_graphs(pa, gpu):
+def test_graph_workspace_grows_outside_captures_and_outlives_graphs(pa, gpu):
     """A partitioned launch recorded in a graph keeps its workspace address: a later, larger
-    launch grows the workspace without freeing the recorded one, and growth inside a capture is
-    an error instead of an allocation from the graph's pool."""
+    recorded launch grows the graphs' workspace without freeing the one already recorded, and
+    growth inside a capture is an error instead of an allocation from the graph's pool."""
     pa.release_decode_workspaces()
     small = cases.make_case(61, [3000, 2000], 2 * 188 + 8)
     d = cases.to_device(small, gpu)
@@ -338,20 +338,22 @@ def test_workspace_is_per_device_grows_outside_captures_and_outlives_graphs(pa, 
         with torch.cuda.graph(g0):
             run_small()
     torch.cuda.synchronize()
-    run_small()                                   # eager warm-up sizes the workspace (1 MiB minimum)
+    with pa.sizing_graph_workspace():
+        run_small()                               # the warm-up before a capture sizes the graphs' workspace (1 MiB minimum)
     torch.cuda.synchronize()
-    ws_first = pa.reserve_decode_workspace(gpu, 1)
+    ws_first = pa.reserve_decode_workspace(gpu, 1, for_graphs=True)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         run_small()
     torch.cuda.synchronize()
-    # a larger launch on the same device: more partials than the first workspace holds
+    # a larger launch for a later graph: more partials than the first workspace holds
     large = cases.make_case(62, [4000] * 24, 24 * 250 + 8)
     dl = cases.to_device(large, gpu)
-    big_out = pa.paged_decode(dl["q"], dl["k_cache"], dl["v_cache"], dl["block_tables"], dl["context_lens"],
-                              dl["scale"], partition_size=64)
+    with pa.sizing_graph_workspace():
+        big_out = pa.paged_decode(dl["q"], dl["k_cache"], dl["v_cache"], dl["block_tables"], dl["context_lens"],
+                                  dl["scale"], partition_size=64)
     torch.cuda.synchronize()
-    ws_second = pa.reserve_decode_workspace(gpu, 1)
+    ws_second = pa.reserve_decode_workspace(gpu, 1, for_graphs=True)
     assert ws_second.numel() > ws_first.numel() and ws_second.data_ptr() != ws_first.data_ptr()
     check(big_out.cpu(), oracle_decode(large), "fp16")
     # fill fresh allocations with garbage: had the first workspace been freed, this would land in it
@@ -365,6 +367,33 @@ def test_workspace_is_per_device_grows_outside_captures_and_outlives_graphs(pa, 
                         dl["scale"], partition_size=64)
         torch.cuda.synchronize()
     del junk
+
+
+def test_partitioned_launches_on_two_streams_do_not_share_partials(pa, gpu):
+    """Eager launches take their workspace per (device, stream): two partitioned launches in flight on
+    different streams of one GPU each merge their own partials."""
+    a = cases.make_case(63, [4000] * 16, 16 * 250 + 8)
+    b = cases.make_case(64, [3500] * 16, 16 * 250 + 8)
+    da, db = cases.to_device(a, gpu), cases.to_device(b, gpu)
+    want_a, want_b = oracle_decode(a), oracle_decode(b)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    outs_a, outs_b = [], []
+    for _ in range(4):
+        outs_a.append(pa.paged_decode(da["q"], da["k_cache"], da["v_cache"], da["block_tables"], da["context_lens"],
+                                      da["scale"], partition_size=128))
+        with torch.cuda.stream(side):
+            outs_b.append(pa.paged_decode(db["q"], db["k_cache"], db["v_cache"], db["block_tables"], db["context_lens"],
+                                          db["scale"], partition_size=128))
+    torch.cuda.synchronize()
+    main_ws = pa.reserve_decode_workspace(gpu, 1)
+    with torch.cuda.stream(side):
+        side_ws = pa.reserve_decode_workspace(gpu, 1)
+    assert main_ws.data_ptr() != side_ws.data_ptr()
+    for o in outs_a:
+        check(o.cpu(), want_a, "fp16")
+    for o in outs_b:
+        check(o.cpu(), want_b, "fp16")
 
 
 # ---- the matrix kernel (q_heads_per_wave = 16; the launch's own choice from a GQA ratio of 3) -------
@@ -398,19 +427,60 @@ def test_matrix_kernel_block_sizes_and_empty_rows(pa, gpu, bs, cache):
         assert float(got[[1, 6]].float().abs().max()) == 0.0       # rows without context come back as zeros
 
 
-@pytest.mark.parametrize("qdt", [torch.float32, torch.bfloat16, torch.float16])
-def test_matrix_kernel_query_dtypes_and_large_scores(pa, gpu, qdt):
+def ramp_keys_along_the_pool(c, lo=0.2, hi=3.0):
+    """Keys grow along the pool (and so, block by block, along the contexts that map it): later tiles hold
+    larger scores than the first one.  An fp8 cache is scaled through its per-token multiplier."""
+    nb, bs = c["k_cache"].shape[0], c["k_cache"].shape[1]
+    ramp = torch.linspace(lo, hi, nb * bs).view(nb, bs)
+    if c["cache_dtype"] == "fp8":
+        c["k_scale"] = c["k_scale"] / ramp
+    else:
+        c["k_cache"] = (c["k_cache"].float() * ramp.view(nb, bs, 1, 1)).to(c["k_cache"].dtype)
+
+
+@pytest.mark.parametrize("qdt,cache", [(torch.float32, "fp16"), (torch.bfloat16, "fp16"), (torch.float16, "fp16"),
+                                       (torch.float16, "fp8"), (torch.bfloat16, "bf16")])
+def test_matrix_kernel_query_dtypes_and_large_scores(pa, gpu, qdt, cache):
     """Scores far from zero (queries and keys of norm ~40): the reference point of the exponentials is
     set by the first tile and moved when a later one outgrows it."""
-    c = cases.make_case(77, [700, 45, 2048, 9], 256, num_heads=32, num_kv_heads=8, q_dtype=qdt)
+    c = cases.make_case(77, [700, 45, 2048, 9], 256, num_heads=32, num_kv_heads=8, q_dtype=qdt, cache=cache)
     c["q"] = (c["q"].float() * 3.5).to(qdt)
-    # keys grow along the context, so later tiles hold the larger scores
-    ramp = torch.linspace(0.2, 3.0, c["k_cache"].shape[0] * c["k_cache"].shape[1]).view(c["k_cache"].shape[0], -1, 1, 1)
-    c["k_cache"] = (c["k_cache"].float() * ramp).to(c["k_cache"].dtype)
+    ramp_keys_along_the_pool(c)
     want = oracle_decode(c)
-    kind = "bf16" if qdt == torch.bfloat16 else "fp16"
+    kind = "fp8" if cache == "fp8" else "bf16" if qdt == torch.bfloat16 else "fp16"
     check(gpu_decode(pa, c, gpu, q_heads_per_wave=16), want, kind)
     check(gpu_decode(pa, c, gpu, q_heads_per_wave=16, partition_size=512, kv_heads_per_wave=2), want, kind)
+
+
+@pytest.mark.parametrize("v_factor", [1e-2, 1e-3])
+@pytest.mark.parametrize("path", ["matrix", "vector"])
+def test_fp8_small_values_behind_an_attention_sink(pa, gpu, path, v_factor):
+    """An fp8 cache whose V is small (per-token amax of 1e-2 .. 1e-3 of the usual) read by rows that put most
+    of their weight on one key of their first tile and spread the rest, ~1e-4 each, over thousands of keys.
+    A kernel that folds 1 / v_scale into the probability before rounding it to fp16 loses that tail
+    (p / v_scale underflows fp16) while the row sum still counts it.  The problem is linear in V, so the
+    fp8 tolerance scales with the factor V was shrunk by."""
+    hq, hkv = (32, 8) if path == "matrix" else (16, 8)
+    lens = [3000, 1500, 4096, 700]
+    c = cases.make_case(311, lens, sum((n + 15) // 16 for n in lens) + 8, num_heads=hq, num_kv_heads=hkv, cache="fp8")
+    g = torch.Generator().manual_seed(312)
+    # the sink: position 0 of every sequence holds a key along the mean query of each KV head's group,
+    # q.k * scale about 9 above the N(0, 1) scores of the other keys
+    gq = hq // hkv
+    qf = c["q"].float().view(len(lens), hkv, gq, 128)
+    k_sink = (0.8 * qf.sum(2)).half()                                   # [batch, hkv, 128]
+    v_sink = torch.randn(len(lens), hkv, 128, generator=g).half()
+    slots = (c["block_tables"][:, 0].long() * 16).to(torch.int32)
+    oracle.store_kv_cache(k_sink, v_sink, c["k_cache"], c["v_cache"], slots, c["k_scale"], c["v_scale"], "fp8")
+    # shrink V through its per-token multiplier: dequantised value = byte / v_scale
+    jitter = 0.5 + 1.5 * torch.rand(c["v_scale"].shape, generator=g)
+    c["v_scale"] = c["v_scale"] / (v_factor * jitter)
+    want = oracle_decode(c)
+    assert want.abs().max() < 20 * v_factor
+    for kw in (dict(), dict(partition_size=512)):
+        got = gpu_decode(pa, c, gpu, q_heads_per_wave=16 if path == "matrix" else 0, **kw)
+        assert not torch.isnan(got).any()
+        torch.testing.assert_close(got.float() / v_factor, want.float() / v_factor, rtol=1e-2, atol=1e-2)
 
 
 def test_matrix_kernel_is_the_choice_for_wide_groups(pa, gpu):
@@ -447,7 +517,8 @@ def test_matrix_kernel_in_a_replayed_graph(pa, gpu, cache):
         pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"], d["scale"],
                         d["k_scale"], d["v_scale"], partition_size=256, out=out2)
 
-    run()                                         # eager warm-up: workspace and kernel attributes
+    with pa.sizing_graph_workspace():
+        run()                                     # warm-up: the graphs' workspace and kernel attributes
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):

@@ -164,3 +164,145 @@ def test_decode_loop_over_the_state_equals_the_prepare_decode_path(pa, gpu, grap
     assert torch.equal(dev.pool.kv_cache_tensor, ref.pool.kv_cache_tensor)
     assert [st.num_tokens(r) for r in rows] == [len(s["token_ids"]) for s in ref.seqs]
     pa.reset_context()
+
+
+def test_state_keeps_prefix_groups_through_admits_and_retires(pa, gpu):
+    """Host side of the group bookkeeping: rebuilt when a row is admitted or retired, never by a step; the
+    device descriptors hold what the host list says."""
+    BS = 16
+    st = pa.DecodeState(8, 32, BS, 1000, device=gpu, num_q_heads=16, num_kv_heads=8, prefix_partition_sizes=(256, 64))
+    assert st.tracks_prefixes and st.prefix_partition_sizes == (256, 64) and st.max_group_rows == 8
+    prompt_a = list(range(100, 117))                      # 17 blocks = 272 tokens
+    prompt_b = list(range(300, 305))                      # 5 blocks = 80 tokens
+    st.admit(prompt_a + [1], 280, 7)
+    st.admit(prompt_b + [2], 82, 7)
+    st.admit(prompt_a + [3], 275, 7)
+    st.admit([900, 901], 20, 7)
+    st.sync_prefix_groups()
+    # prompt a shares one partition of 256 (or four of 64: no more tokens), prompt b has one row only
+    assert st.prefix_groups_host == [([0, 2], 256)] and st.prefix_partition_size == 256
+    st.admit(prompt_b + [4], 85, 7)                       # row 4: b's second sample shares 64 tokens
+    st.sync_prefix_groups()
+    # 64-token partitions now save 256 + 64 tokens of reads against 256 with the coarse size: the finer size wins
+    assert st.prefix_partition_size == 64 and st.prefix_groups_host == [([0, 2], 256), ([1, 4], 64)]
+    pg = st.prefix_groups(5)
+    assert (pg.num_groups, pg.max_group_rows, pg.max_shared_partitions, pg.partition_size) == (2, 2, 4, 64)
+    torch.cuda.synchronize()
+    assert pg.group_desc[:2].tolist() == [[0, 2, 4, 0], [2, 2, 1, 0]] and int(pg.group_desc[2:].abs().sum()) == 0
+    assert pg.group_rows[:4].tolist() == [0, 2, 1, 4] and pg.row_skip.tolist() == [4, 1, 4, 0, 1]
+    for _ in range(3):                                    # steps change nothing
+        st.step(None)
+        assert not st._groups_dirty and st.prefix_groups_host == [([0, 2], 256), ([1, 4], 64)]
+    st.retire(0)
+    assert st.prefix_groups(5).groups == [([1, 4], 64)]
+    torch.cuda.synchronize()
+    assert st._row_skip.tolist()[:5] == [0, 1, 0, 0, 1]
+    st.retire(4)
+    assert st.prefix_groups(5) is None and st.prefix_partition_size is None
+    torch.cuda.synchronize()
+    assert int(st._groups_dev.abs().sum()) == 0          # nothing on the device names a row any more
+    # the capacity view a graph is recorded over
+    cap = st.prefix_groups(8, 256, for_graph=True)
+    assert (cap.num_groups, cap.max_group_rows, cap.max_shared_partitions, cap.partition_size) == (4, 8, 2, 256)
+    # a state that was not told the head layout keeps no groups
+    assert pa.DecodeState(4, 8, BS, 100, device=gpu).prefix_groups(4) is None
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_forked_samples_decode_through_shared_prefix_groups(pa, gpu, graphs):
+    """Samples forked from prefilled prompts (KVCacheManager.fork_sequence, copy-on-write of the shared last
+    block), interleaved rows, a retirement and a late fork: the decode loop over DecodeState takes the
+    shared-prefix launch (recorded in a graph or eager) whenever the state holds a group, and its logits
+    equal those of the same sequences decoded from private, unshared blocks through prepare_decode."""
+    from test_gpu_model import Session, small_model
+    BS = 16
+    model = small_model(pa, seed=23)                  # 4 query / 2 KV heads: up to 8 rows per group
+    ref = Session(pa, model, gpu, num_blocks=128)     # every sequence owns all its blocks
+    ref.runner.config.share_prefix_decode = False
+    dev = Session(pa, model, gpu, num_blocks=128, graphs=None)
+    dev.runner.config.enable_cuda_graph = graphs
+    mgr = pa.KVCacheManager(dev.pool, BS)
+    g = torch.Generator().manual_seed(24)
+    prompts = {"a": torch.randint(0, 512, (70,), generator=g).tolist(),     # 4 full blocks + 6 tokens
+               "b": torch.randint(0, 512, (40,), generator=g).tolist(),     # 2 full blocks + 8 tokens
+               "c": torch.randint(0, 512, (50,), generator=g).tolist()}
+    # prefill each prompt once on the device path, from the manager's blocks
+    first = {}
+    for name, toks in prompts.items():
+        table = mgr.allocate_for_sequence((name, 0), len(toks)).get_physical_block_ids()
+        ids, pos = dev.runner.prepare_prefill([{"token_ids": toks, "block_table": table, "num_cached_tokens": 0,
+                                                "num_scheduled_tokens": len(toks)}])
+        first[name] = int(dev.runner.run(ids, pos, is_prefill=True)[-1].argmax())
+    order = [("a", 0), ("b", 0), ("a", 1), ("c", 0), ("a", 2), ("b", 1), ("a", 3)]     # samples interleaved
+    for name, s in order:
+        if s:
+            mgr.fork_sequence((name, 0), (name, s))
+    st = pa.DecodeState(8, 8, BS, dev.pool.num_blocks, device=gpu, num_q_heads=4, num_kv_heads=2,
+                        prefix_partition_sizes=(64, 32))
+    seq_of_row, ref_of_row, tokens = {}, {}, {}
+    for name, s in order:
+        tok = (first[name] + 17 * s) % 512                               # the samples diverge at once
+        row = st.admit(mgr.get_block_table((name, s)), len(prompts[name]), tok)
+        seq_of_row[row], tokens[row] = (name, s), tok
+        ref.add(prompts[name])
+        ref_of_row[row] = len(ref.seqs) - 1
+    ref.prefill()
+    st.sync_prefix_groups()
+    assert st.prefix_groups_host == [([0, 2, 4, 6], 64), ([1, 5], 32)] and st.prefix_partition_size == 32
+    if graphs:
+        dev.runner.capture_decode_state_graphs(st, [8])
+    next_dev = None
+    for step in range(24):
+        if step == 8:                      # a sample of prompt a leaves: its group shrinks
+            mgr.free_sequence(seq_of_row[2])
+            st.retire(2)
+            del seq_of_row[2]
+        if step == 12:                     # a late fork of b's first sample (generated tokens included) takes the free row
+            parent_row = next(r for r, sq in seq_of_row.items() if sq == ("b", 0))
+            mgr.fork_sequence(("b", 0), ("b", 9))
+            history = ref.seqs[ref_of_row[parent_row]]["token_ids"]
+            row = st.admit(mgr.get_block_table(("b", 9)), len(history), 5)
+            assert row == 2
+            seq_of_row[2], tokens[2] = ("b", 9), 5
+            ref.add(list(history))
+            ref.prefill()
+            ref_of_row[2] = len(ref.seqs) - 1
+            st.sync_prefix_groups()
+            assert ([1, 2, 5], 32) in st.prefix_groups_host
+        # the manager makes room for every row's new token: a new block, or a private copy of a shared last block
+        grants = {}
+        for row, sq in seq_of_row.items():
+            before = mgr.get_block_table(sq)
+            assert mgr.append_token(sq)
+            after = mgr.get_block_table(sq)
+            if len(after) > len(before) or after[-1] != before[-1]:
+                grants[row] = after[-1]
+        mgr.apply_copies()
+        st.step(grants or None, next_dev)
+        got = dev.runner.run_decode_state(st)
+        # the same step on private blocks
+        ref_tokens = [0] * len(ref.seqs)
+        for row, tok in tokens.items():
+            ref_tokens[ref_of_row[row]] = tok
+        want = ref.decode(ref_tokens)
+        for row in seq_of_row:
+            torch.testing.assert_close(got[row].float().cpu(), want[ref_of_row[row]].float().cpu(), rtol=2e-3, atol=2e-3)
+        next_dev = pa.sample_tokens(got, temperature=0.0)
+        picked = next_dev.tolist()
+        for row in seq_of_row:
+            tokens[row] = picked[row]
+    stats = dev.runner.decode_state_stats
+    if graphs:
+        assert stats["shared_prefix_graph"] == 24 and stats["plain_graph"] == 0 and stats["eager"] == 0
+    else:
+        assert stats["eager"] == 24
+    # without the last group the plain graph takes over
+    for row, sq in list(seq_of_row.items()):
+        if sq[0] in ("a", "b") and row != 0:
+            st.retire(row)
+    st.sync_prefix_groups()
+    assert st.prefix_partition_size is None
+    st.step(None, next_dev)
+    dev.runner.run_decode_state(st)
+    assert stats["plain_graph" if graphs else "eager"] == (1 if graphs else 25)
+    pa.reset_context()

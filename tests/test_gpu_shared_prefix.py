@@ -69,15 +69,107 @@ def test_ragged_groups_loners_and_partial_partitions(pa, gpu):
     check(shared_decode(pa, c, gpu, groups64, partition_size=64, waves=8), want, "fp16")
 
 
-def test_fourth_benchmark_configuration(pa, gpu):
-    """32 prompts x 8 samples, 1024 shared tokens, private suffixes (reduced to 6 prompts for the oracle)."""
-    gen = torch.Generator().manual_seed(1004)
-    suf = torch.randint(64, 513, (48,), generator=gen).tolist()
-    lens = [1024 + x for x in suf]
-    c = cases.make_case(1004, lens, 6 * 64 + sum((x + 15) // 16 for x in suf) + 16, shared_prefix=(8, 64))
-    groups = pa.find_prefix_groups(host_tables(c), lens, 16, 16, 8)
-    assert groups == [(8 * i, 8, 1024) for i in range(6)]
-    check(shared_decode(pa, c, gpu, groups), oracle_decode(c), "fp16")
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_fourth_benchmark_configuration_at_full_size(pa, gpu, cache):
+    """32 prompts x 8 samples = 256 rows, 1024 shared tokens per prompt, private suffixes U[64, 512]: the
+    shared-prefix launch on the whole batch, groups and partition size from the finder, against the
+    oracle - and the same rows shuffled, so that no group's rows are neighbours."""
+    c = cases.config4(cache=cache)
+    lens = c["context_lens"].tolist()
+    tables = host_tables(c)
+    pg = pa.prepare_prefix_groups(tables, lens, 16, 16, 8, gpu)
+    assert pg.partition_size == 1024 and pg.groups == [(list(range(8 * i, 8 * i + 8)), 1024) for i in range(32)]
+    assert pg.group_rows is None
+    want = oracle_decode(c)
+    d = cases.to_device(c, gpu)
+    got = pa.paged_decode_shared_prefix(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                                        d["scale"], None, d["k_scale"], d["v_scale"], descriptors=pg)
+    torch.cuda.synchronize()
+    check(got.cpu(), want, cache)
+    # finer partitions (more of them shared: 4 x 256 per prompt)
+    check(shared_decode(pa, c, gpu, pa.find_prefix_groups(tables, lens, 16, 16, 8, 256), partition_size=256), want, cache)
+    # the rows in a random order: groups are lists of rows
+    perm = torch.randperm(256, generator=torch.Generator().manual_seed(4)).tolist()
+    far = pa.prepare_prefix_groups([tables[i] for i in perm], [lens[i] for i in perm], 16, 16, 8, gpu, anywhere=True)
+    assert far.partition_size == 1024 and far.num_groups == 32 and far.group_rows is not None
+    inv = {old: new for new, old in enumerate(perm)}
+    assert sorted(far.groups) == sorted((sorted(inv[r] for r in range(8 * i, 8 * i + 8)), 1024) for i in range(32))
+    idx = torch.tensor(perm, device=gpu)
+    got = pa.paged_decode_shared_prefix(d["q"][idx].contiguous(), d["k_cache"], d["v_cache"],
+                                        d["block_tables"][idx].contiguous(), d["context_lens"][idx].contiguous(),
+                                        d["scale"], None, d["k_scale"], d["v_scale"], descriptors=far)
+    torch.cuda.synchronize()
+    check(got.cpu(), want[perm], cache)
+
+
+@pytest.mark.parametrize("hq,hkv", [(16, 8), (32, 8)])
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_groups_of_rows_anywhere_in_the_batch(pa, gpu, cache, hq, hkv):
+    """Samples of three prompts interleaved with each other and with rows of their own; padding groups of no
+    partitions between the real ones (what a recorded launch at full capacity holds)."""
+    group = 16 // (hq // hkv)
+    lens = [300 + 7 * i for i in range(3 * group)] + [90, 500]
+    pool = sum((n + 15) // 16 for n in lens) + 16
+    c = cases.make_case(900 + hq, lens, pool, num_heads=hq, num_kv_heads=hkv, cache=cache, shared_prefix=None)
+    tb = c["block_tables"]
+    for p_ in range(3):
+        for m in range(1, group):
+            tb[p_ * group + m, :16] = tb[p_ * group, :16]            # 256 shared tokens per prompt
+    order = torch.randperm(len(lens), generator=torch.Generator().manual_seed(hq)).tolist()
+    for key in ("q", "block_tables", "context_lens"):
+        c[key] = c[key][order].contiguous()
+    lens = c["context_lens"].tolist()
+    want = oracle_decode(c)
+    groups = pa.find_prefix_groups_anywhere(host_tables(c), lens, 16, hq, hkv, 128)
+    assert len(groups) == 3 and all(len(rows) == group and tokens == 256 for rows, tokens in groups)
+    assert any(rows != list(range(rows[0], rows[0] + group)) for rows, _ in groups)
+    check(shared_decode(pa, c, gpu, groups, partition_size=128), want, cache)
+    # the descriptors a recorded graph uses: more groups than there are, the spare ones empty
+    pg = pa.shared_prefix_descriptors(groups, len(lens), gpu, 128)
+    desc = torch.zeros(8, 4, dtype=torch.int32, device=gpu)
+    desc[1], desc[4], desc[6] = pg.group_desc[0], pg.group_desc[1], pg.group_desc[2]
+    padded = pa.PrefixGroups(128, desc, pg.group_rows, pg.row_skip, 8, group, 5, 0)
+    d = cases.to_device(c, gpu)
+    got = pa.paged_decode_shared_prefix(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                                        d["scale"], None, d["k_scale"], d["v_scale"], descriptors=padded)
+    torch.cuda.synchronize()
+    check(got.cpu(), want, cache)
+
+
+def test_corrupt_descriptors_do_not_fault(pa, gpu, monkeypatch):
+    """Everything the kernel reads from the descriptors is clamped before it indexes anything: rows outside
+    the batch, more rows than the operand holds, a row list index past the list, negative skips.  The launch
+    must come back (with wrong numbers for the rows involved), and the checker must name the damage."""
+    lens = [600, 610, 620, 630, 300]
+    c = cases.make_case(6, lens, 220, shared_prefix=(4, 32))
+    d = cases.to_device(c, gpu)
+    good = pa.shared_prefix_descriptors([([0, 1, 2, 3], 512)], 5, gpu, 128)
+    want = oracle_decode(c)
+    for damage in ("rows", "row_index", "first", "skip"):
+        desc, rows, skip = good.group_desc.clone(), good.group_rows, good.row_skip.clone()
+        rows = torch.tensor([0, 1, 2, 3, 0], dtype=torch.int32, device=gpu)
+        desc[0, 0] = 0
+        if damage == "rows":
+            desc[0, 1] = 4000
+        elif damage == "row_index":
+            rows[2] = 70000
+        elif damage == "first":
+            desc[0, 0] = 123456
+        else:
+            skip[4] = -7
+        bad = pa.PrefixGroups(128, desc, rows, skip, 1, 4, 4, 0)
+        out = pa.paged_decode_shared_prefix(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                                            d["scale"], None, descriptors=bad)
+        torch.cuda.synchronize()
+        assert out.shape == d["q"].shape
+        if damage == "skip":
+            check(out.cpu(), want, "fp16")           # a negative skip is read as no skip: still the right answer
+        if damage in ("rows", "row_index", "first"):
+            monkeypatch.setenv("PA_DEBUG_TABLES", "1")
+            with pytest.raises(RuntimeError, match="shared table entries differ|rows too short|outside the groups"):
+                pa.paged_decode_shared_prefix(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"],
+                                              d["scale"], None, descriptors=bad)
+            monkeypatch.delenv("PA_DEBUG_TABLES")
 
 
 def test_descriptor_check_and_refusals(pa, gpu, monkeypatch):
@@ -112,7 +204,7 @@ def test_attention_layers_take_the_groups_from_the_context(pa, gpu, layer):
     att = getattr(pa, layer)(16, 8, 128)
     att.k_cache, att.v_cache = d["k_cache"], d["v_cache"]
     pg = pa.prepare_prefix_groups(host_tables(c), lens, 16, 16, 8, gpu)
-    assert pg["groups"] == [(0, 8, 512)]
+    assert pg.groups == [(list(range(8)), 512)] and pg.partition_size == 512
     new_k = torch.zeros(10, 8, 128, dtype=torch.float16, device=gpu)
     outs = {}
     for name, groups in (("shared", pg), ("plain", None)):

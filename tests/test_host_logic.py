@@ -120,23 +120,56 @@ def test_find_prefix_groups(pa):
     assert f([], [], 16, 16, 8) == []
 
 
+def test_find_prefix_groups_anywhere(pa):
+    f = pa.find_prefix_groups_anywhere
+    shared = list(range(100, 140))                       # 40 blocks = 640 tokens
+    other = list(range(700, 716))                        # 16 blocks = 256 tokens
+    # samples of two prompts interleaved, a loner between them, a row that shares only half of the first prompt
+    rows = [shared + [1], other + [2], shared + [3], [900, 901], other + [4], shared[:20] + [5], shared + [6]]
+    lens = [650, 260, 650, 20, 260, 330, 650]
+    assert f(rows, lens, 16, 16, 8, 128) == [([0, 2, 6], 640), ([1, 4], 256)]
+    # the row that shares half the prompt stays out: three rows sharing 512 tokens save more reads than four sharing 256
+    assert f(rows, lens, 16, 16, 8, 256) == [([0, 2, 6], 512), ([1, 4], 256)]
+    # ... and is taken in where that is what saves more
+    assert f(rows[:1] + rows[5:6] + rows[2:3], [650, 330, 650], 16, 16, 8, 64) == [([0, 2], 640)]
+    assert f(rows[:1] + rows[5:6], [650, 330], 16, 16, 8, 64) == [([0, 1], 320)]
+    # the rows argument names the batch rows the tables belong to
+    assert f(rows[:3], lens[:3], 16, 16, 8, 128, rows=[4, 9, 11]) == [([4, 11], 640)]
+    # four query heads per KV head: at most four rows per group
+    assert f([shared + [i] for i in range(6)], [650] * 6, 16, 32, 8, 128) == [([0, 1, 2, 3], 640), ([4, 5], 640)]
+    # a context shorter than a partition shares nothing; empty tables are skipped
+    assert f([shared, shared, []], [100, 650, 0], 16, 16, 8, 128) == []
+    assert f([], [], 16, 16, 8) == []
+    # a partition size the blocks do not divide finds nothing (and does not divide by zero)
+    assert pa.find_prefix_groups([shared, shared], [650, 650], 512, 16, 8, 256) == []
+
+
 def test_shared_prefix_descriptors_and_context_field(pa):
-    desc, skip, max_rows, max_parts, min_skip = pa.shared_prefix_descriptors([(0, 3, 512), (5, 2, 1024)], 8, "cpu", 256)
-    assert desc.dtype == torch.int32 and desc.tolist() == [[0, 3, 2, 0], [5, 2, 4, 0]]
-    assert skip.tolist() == [2, 2, 2, 0, 0, 4, 4, 0] and (max_rows, max_parts, min_skip) == (3, 4, 0)
-    assert pa.shared_prefix_descriptors([(0, 2, 512)], 2, "cpu", 256)[4] == 2        # every row skips two
+    pg = pa.shared_prefix_descriptors([(0, 3, 512), (5, 2, 1024)], 8, "cpu", 256)
+    assert pg.group_desc.dtype == torch.int32 and pg.group_desc.tolist() == [[0, 3, 2, 0], [5, 2, 4, 0]]
+    assert pg.group_rows is None                          # consecutive rows need no list
+    assert pg.row_skip.tolist() == [2, 2, 2, 0, 0, 4, 4, 0]
+    assert (pg.num_groups, pg.max_group_rows, pg.max_shared_partitions, pg.min_row_skip, pg.batch) == (2, 3, 4, 0, 8)
+    assert pa.shared_prefix_descriptors([(0, 2, 512)], 2, "cpu", 256).min_row_skip == 2        # every row skips two
+    # rows anywhere in the batch: the descriptor's first entry indexes the row list
+    pg = pa.shared_prefix_descriptors([([1, 4, 6], 512), ([0, 7], 256)], 8, "cpu", 256)
+    assert pg.group_desc.tolist() == [[0, 3, 2, 0], [3, 2, 1, 0]]
+    assert pg.group_rows.tolist()[:5] == [1, 4, 6, 0, 7]
+    assert pg.row_skip.tolist() == [1, 2, 0, 0, 2, 0, 2, 1]
     with pytest.raises(RuntimeError, match="outside the batch"):
         pa.shared_prefix_descriptors([(7, 2, 512)], 8, "cpu", 256)
     assert pa.prepare_prefix_groups([[1, 2], [3, 4]], [32, 32], 16, 16, 8, "cpu", 32) is None
     # no partition size given: the coarsest of 2048 / 1024 / 512 / 256 that keeps 90 % of the savings
     shared = list(range(100, 164))                       # 64 blocks = 1024 tokens
     auto = pa.prepare_prefix_groups([shared[:40] + [7], shared[:40] + [8]], [650, 650], 16, 16, 8, "cpu")
-    assert auto["partition_size"] == 512 and auto["groups"] == [(0, 2, 512)]
+    assert auto.partition_size == 512 and auto.groups == [([0, 1], 512)]
     auto = pa.prepare_prefix_groups([shared + [7], shared + [8]], [1030, 1030], 16, 16, 8, "cpu")
-    assert auto["partition_size"] == 1024 and auto["groups"] == [(0, 2, 1024)]
+    assert auto.partition_size == 1024 and auto.groups == [([0, 1], 1024)]
     assert pa.prepare_prefix_groups([shared[:10] + [7], shared[:10] + [8]], [170, 170], 16, 16, 8, "cpu") is None
     pg = pa.prepare_prefix_groups([[1, 2, 9], [1, 2, 8]], [40, 40], 16, 16, 8, "cpu", 32)
-    assert pg["groups"] == [(0, 2, 32)] and pg["partition_size"] == 32
+    assert pg.groups == [([0, 1], 32)] and pg.partition_size == 32
+    far = pa.prepare_prefix_groups([[1, 2, 9], [5, 5, 5], [1, 2, 8]], [40, 40, 40], 16, 16, 8, "cpu", 32, anywhere=True)
+    assert far.groups == [([0, 2], 32)] and far.group_rows.tolist()[:2] == [0, 2]
     pa.set_context(False, context_lens=torch.ones(2, dtype=torch.int32), prefix_groups=pg)
     assert pa.get_context().prefix_groups is pg
     pa.reset_context()

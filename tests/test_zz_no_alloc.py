@@ -42,13 +42,41 @@ def _both(lib, gpu, c, psize, H=H):
 def test_two_calls_in_a_row_second_one_smaller(lib, gpu, cache):
     big = cases.make_case(901, [3000, 517, 4096, 1, 2222, 1025], 6 * 256 + 16, cache=cache)
     small = cases.make_case(902, [700, 90], 64, cache=cache)
-    # memory activity between the calls must not disturb the array either
     allocated_before = torch.cuda.memory_allocated(gpu)
     for c, psize in ((big, 256), (small, 512)):
         got, want = _both(lib, gpu, c, psize)
         assert not torch.isnan(got).any()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.cuda.memory_allocated(gpu) == allocated_before
+
+
+def test_the_entry_point_takes_no_device_memory(lib, gpu):
+    """torch's own counters cannot see a hipMalloc made inside the library, so the device-wide free bytes
+    are read around the calls (hipMemGetInfo): with every input, output and the comparison workspace
+    allocated beforehand, and the library's array resident since it was loaded, calls of the entry point -
+    partitioned, over several shapes - must leave the free bytes where they were."""
+    cs = [cases.make_case(906, [3000, 517, 4096, 1, 2222, 1025], 6 * 256 + 16),
+          cases.make_case(907, [700, 90], 64, cache="fp8")]
+    ds = [cases.to_device(c, gpu) for c in cs]
+    outs = [torch.empty(d["q"].shape, dtype=torch.float16, device=gpu) for d in ds]
+    stream = torch.cuda.current_stream(gpu).cuda_stream
+    def run_all():
+        for c, d, o in zip(cs, ds, outs):
+            for psize in (256, 128, 1024):
+                parts = (d["block_tables"].shape[1] * BS + psize - 1) // psize
+                assert lib.pa_decode_noalloc(*_args(d, c, o), psize, parts, 0, 0, 0, stream) == 0, lib.pa_last_error()
+        torch.cuda.synchronize()
+
+    # a first call per launch shape: what the runtime sets up once per kernel and process (code object,
+    # kernel attributes, the symbol lookup) is not what this test is about
+    run_all()
+    free_before, _total = torch.cuda.mem_get_info(gpu)
+    torch_before = torch.cuda.memory_reserved(gpu)
+    for _ in range(3):
+        run_all()
+    free_after, _total = torch.cuda.mem_get_info(gpu)
+    assert torch.cuda.memory_reserved(gpu) == torch_before       # torch itself took nothing in between ...
+    assert free_after == free_before, (free_before, free_after)   # ... and neither did anyone else on the device
 
 
 def test_wide_query_groups_take_the_matrix_kernel_through_the_same_entry_point(lib, gpu):
