@@ -487,14 +487,15 @@ def _debug_tables():
 # many workgroups it hosts (about 1.3 x its 1/256 share).  Workgroups are dealt to CUs in rounds,
 # so the launch lasts as long as its busiest CU needs: 288 equal workgroups on 256 CUs make two
 # rounds, not 1.125.  The context is split where the larger of the two bounds, plus about 2 us per
-# round of workgroups and 5 us + 0.25 us per partition for the merge pass, is smallest.  The rates
-# are measurements on an MI355X (batch 4..128, contexts 2k..32k, fp16 and fp8 caches).
+# round of workgroups and 3 us + 0.03 us per partition for the merge pass, is smallest.  The rates
+# are fitted to a sweep of every split on an MI355X (batch 1..128, contexts 2k..32k, fp16 and fp8
+# caches, streaming loads): the pick is within 1.5 % of the best measured split on average, 7 % at worst.
 _MIN_AUTO_PARTITION = 256          # tokens
 _MAX_AUTO_PARTITIONS = 128
-_HBM_BYTES_PER_NS = 6050.0
-_CU_BYTES_PER_NS = {2: 31.0, 1: 22.0}      # by cache element size: fp8 rows cost more arithmetic per byte
+_HBM_BYTES_PER_NS = 6800.0
+_CU_BYTES_PER_NS = {2: 28.0, 1: 25.0}      # by cache element size
 _ROUND_NS = 2000.0
-_MERGE_NS = (5000.0, 250.0)        # fixed, per partition (the pass itself and the partials it re-reads)
+_MERGE_NS = (3000.0, 30.0)         # fixed, per partition (the pass itself and the partials it re-reads)
 _DEFAULT_COMPUTE_UNITS = 256
 MATRIX_PATH_FROM_RATIO = 3         # GQA ratio from which pa_decode multiplies on the matrix cores (up to 16 query heads per workgroup)
 _CU_COUNT = {}

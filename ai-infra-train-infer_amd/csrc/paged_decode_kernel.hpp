@@ -78,6 +78,7 @@ struct DecodeParams {
   const int32_t* group_rows;   // batch rows of the groups, one run per group; nullptr: a group's rows are consecutive
   int group_rows_len;          // entries of group_rows
   const int32_t* row_skip;     // [batch]: leading partitions of the row that its group computes
+  int num_groups;              // entries of group_desc
   int num_prefix_wgs;          // groups x prefix_parts x inner
   int prefix_parts;            // most shared partitions of any group
   int suffix_parts;            // most own partitions of any row

@@ -282,7 +282,7 @@ inline int plan_decode(const char* who, const void* q, int q_dtype, int64_t q_to
   p.group_rows = nullptr;
   p.group_rows_len = 0;
   p.row_skip = nullptr;
-  p.num_prefix_wgs = p.prefix_parts = p.suffix_parts = 0;
+  p.num_groups = p.num_prefix_wgs = p.prefix_parts = p.suffix_parts = 0;
   int64_t wgs = batch * max_partitions * p.inner;
   if (shared) {
     const int64_t prefix_wgs = shared->num_groups * shared->max_shared_partitions * p.inner;
@@ -292,6 +292,7 @@ inline int plan_decode(const char* who, const void* q, int q_dtype, int64_t q_to
     p.group_rows = shared->group_rows;
     p.group_rows_len = (int)shared->num_group_rows;
     p.row_skip = shared->row_skip;
+    p.num_groups = (int)shared->num_groups;
     p.num_prefix_wgs = (int)prefix_wgs;
     p.prefix_parts = (int)shared->max_shared_partitions;
     p.suffix_parts = (int)shared->max_own_partitions;

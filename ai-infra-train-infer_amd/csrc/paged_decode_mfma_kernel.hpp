@@ -168,12 +168,17 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   if (p.group_desc) {
     // Descriptors come from device memory: everything read from them is brought into range before
     // it is used as an index, so that a corrupt descriptor gives wrong numbers, never a fault.
+    // Workgroups that find nothing to do (a group with fewer shared partitions than the launch is sized
+    // for, a padding group, a row with fewer partitions of its own) should sit together in the grid, not
+    // between working ones: interleaved, 2048 of them cost the fourth benchmark configuration 32 us,
+    // in one run at the end of a region next to nothing.  So both regions walk their partition index
+    // last: all first partitions, then all second ones, ...
     int x = blockIdx.x;
     if (x < p.num_prefix_wgs) {
       in = x % p.inner;
       const int u = x / p.inner;
-      part = u % p.prefix_parts;
-      const int32_t* desc = p.group_desc + 4 * (u / p.prefix_parts);
+      part = u / p.num_groups;
+      const int32_t* desc = p.group_desc + 4 * (u % p.num_groups);
       if (part >= desc[2]) return;
       members = min(desc[1], NHC / max(gq, 1));
       if (members < 1) return;
@@ -191,8 +196,8 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       x -= p.num_prefix_wgs;
       in = x % p.inner;
       const int u = x / p.inner;
-      b = u / p.suffix_parts;
-      part = min(max(p.row_skip[b], 0), p.max_partitions) + u % p.suffix_parts;
+      b = u % p.batch;
+      part = min(max(p.row_skip[b], 0), p.max_partitions) + u / p.batch;
       if (part >= p.max_partitions) return;
     }
   } else {

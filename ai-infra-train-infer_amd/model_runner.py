@@ -99,8 +99,9 @@ class DecodeState:
         self._stage = [[torch.full((max_batch,), -1, dtype=torch.int32).pin_memory(), None] for _ in range(2)]
         self._turn = 0
         self._fresh_rows = set()                        # host copy of the same
-        self._lens = [0] * max_batch                    # tokens in the cache, per row (0 = free)
-        self._tables = [[] for _ in range(max_batch)]   # block ids, per row
+        self._lens = np.zeros(max_batch, dtype=np.int64)    # tokens in the cache, per row (0 = free)
+        self._ntab = np.zeros(max_batch, dtype=np.int64)    # block ids held, per row
+        self._tables = [[] for _ in range(max_batch)]       # the block ids themselves
         # ---- rows that share prefixes ---------------------------------------------------------------
         self._heads = (int(num_q_heads), int(num_kv_heads)) if num_q_heads and num_kv_heads else None
         self.max_group_rows = 16 // max(1, self._heads[0] // self._heads[1]) if self._heads else 0
@@ -122,16 +123,14 @@ class DecodeState:
     @property
     def rows_in_use(self) -> int:
         """One past the highest active row."""
-        for r in range(self.max_batch - 1, -1, -1):
-            if self._lens[r] > 0:
-                return r + 1
-        return 0
+        used = np.flatnonzero(self._lens)
+        return int(used[-1]) + 1 if used.size else 0
 
     def active_rows(self) -> List[int]:
-        return [r for r in range(self.max_batch) if self._lens[r] > 0]
+        return np.flatnonzero(self._lens).tolist()
 
     def num_tokens(self, row: int) -> int:
-        return self._lens[row]
+        return int(self._lens[row])
 
     def admit(self, block_table: List[int], num_cached_tokens: int, next_token: int) -> int:
         """Give a prefilled sequence (its `num_cached_tokens` tokens are in the cache, `next_token`
@@ -140,10 +139,10 @@ class DecodeState:
             raise RuntimeError("DecodeState.admit: a sequence enters decode with at least one cached token")
         if len(block_table) > self.max_blocks or len(block_table) * self.block_size < num_cached_tokens:
             raise RuntimeError("DecodeState.admit: block table does not fit the state or the tokens")
-        try:
-            row = self._lens.index(0)
-        except ValueError:
-            raise RuntimeError("DecodeState.admit: all %d rows are in use" % self.max_batch) from None
+        free = np.flatnonzero(self._lens == 0)
+        if not free.size:
+            raise RuntimeError("DecodeState.admit: all %d rows are in use" % self.max_batch)
+        row = int(free[0])
         host_row = torch.full((self.max_blocks,), -1, dtype=torch.int32)
         host_row[:len(block_table)] = torch.tensor(block_table, dtype=torch.int32)
         self.block_tables[row].copy_(host_row.pin_memory(), non_blocking=True)
@@ -153,6 +152,7 @@ class DecodeState:
         self._fresh_rows.add(row)
         self._lens[row] = int(num_cached_tokens)
         self._tables[row] = list(block_table)
+        self._ntab[row] = len(block_table)
         self._groups_dirty = self.tracks_prefixes
         return row
 
@@ -160,7 +160,7 @@ class DecodeState:
         """Free a row; returns the block ids the sequence held."""
         self.context_lens[row].fill_(0)
         self._fresh_rows.discard(row)
-        blocks, self._tables[row], self._lens[row] = self._tables[row], [], 0
+        blocks, self._tables[row], self._lens[row], self._ntab[row] = self._tables[row], [], 0, 0
         self._groups_dirty = self.tracks_prefixes
         return blocks
 
@@ -181,7 +181,7 @@ class DecodeState:
         self._groups_dirty = False
         active = self.active_rows()
         tables = [self._tables[r] for r in active]
-        lens = [self._lens[r] for r in active]
+        lens = [int(self._lens[r]) for r in active]
         hq, hkv = self._heads
 
         def find(size):
@@ -231,8 +231,8 @@ class DecodeState:
     def rows_needing_block(self) -> List[int]:
         """Active rows whose next token opens a block they do not have yet."""
         bs = self.block_size
-        return [r for r in range(self.max_batch)
-                if self._lens[r] > 0 and self._lens[r] % bs == 0 and self._lens[r] // bs >= len(self._tables[r])]
+        lens = self._lens
+        return np.flatnonzero((lens > 0) & (lens % bs == 0) & (lens // bs >= self._ntab)).tolist()
 
     def step(self, new_blocks: Optional[Dict[int, int]] = None, next_tokens: Optional[torch.Tensor] = None):
         """Advance every active row by one token.  new_blocks: {row: block id} for the rows of
@@ -243,21 +243,23 @@ class DecodeState:
         from . import _native
         lib = _native.load()
         self.sync_prefix_groups()
-        n = self.rows_in_use
         if next_tokens is not None:
             next_tokens = next_tokens.reshape(-1)
             if not next_tokens.is_cuda or next_tokens.dtype != torch.long or not next_tokens.is_contiguous():
                 raise RuntimeError("DecodeState.step: next_tokens must be a contiguous int64 GPU tensor")
-            fed = [r for r in range(n) if self._lens[r] > 0 and r not in self._fresh_rows]
-            if fed and fed[-1] >= next_tokens.numel():
-                raise RuntimeError("DecodeState.step: next_tokens has no entry for row %d" % fed[-1])
+            # the highest row that takes its input from next_tokens (active, not admitted since the last step)
+            last_fed = next((r for r in np.flatnonzero(self._lens)[::-1].tolist() if r not in self._fresh_rows), -1)
+            if last_fed >= next_tokens.numel():
+                raise RuntimeError("DecodeState.step: next_tokens has no entry for row %d" % last_fed)
             if next_tokens.numel() < self.max_batch:      # the kernel indexes it by row
                 padded = torch.zeros(self.max_batch, dtype=torch.long, device=next_tokens.device)
                 padded[:next_tokens.numel()] = next_tokens
                 next_tokens = padded
-        missing = [r for r in self.rows_needing_block() if not new_blocks or r not in new_blocks]
-        if missing:
-            raise RuntimeError("DecodeState.step: rows %s need a new block" % missing)
+        need = self.rows_needing_block()
+        if need:
+            missing = [r for r in need if not new_blocks or r not in new_blocks]
+            if missing:
+                raise RuntimeError("DecodeState.step: rows %s need a new block" % missing)
         new_ptr = None
         if new_blocks:
             host, event = self._stage[self._turn]
@@ -273,6 +275,7 @@ class DecodeState:
                     self._tables[row][col] = int(block)          # copy-on-write: a private copy replaces it
                 else:
                     self._tables[row].append(int(block))
+                    self._ntab[row] += 1
             self._new_blocks.copy_(host, non_blocking=True)
             done = torch.cuda.Event()
             done.record()
@@ -287,9 +290,7 @@ class DecodeState:
                                    self._fresh.data_ptr(), self.max_batch, self.max_blocks,
                                    self.block_size, self.num_blocks, stream)
         _native.check(rc, "pa_decode_advance")
-        for r in range(self.max_batch):
-            if self._lens[r] > 0:
-                self._lens[r] += 1
+        self._lens[self._lens > 0] += 1
         self._fresh_rows.clear()
 
     def set_context(self, batch: Optional[int] = None, share_prefixes: bool = True,
@@ -327,6 +328,7 @@ class ModelRunner:
         self._graph_batch_sizes: List[int] = []
         self._state_graphs: Dict[Tuple[int, int, Optional[int]], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._hf_model: Optional[torch.nn.Module] = None
+        self._state_graph_lookup: Dict[Tuple[int, int, Optional[int]], object] = {}
         self._prefix_groups_kept = None          # (signature of the batch, PrefixGroups or None) of the last decode step
         # how run_decode_state ran its steps: replays of a graph recorded over the shared-prefix launch,
         # replays of a plain graph, eager forwards
@@ -741,8 +743,20 @@ class ModelRunner:
                 if self._graph_pool is None:
                     self._graph_pool = graph.pool()
                 self._state_graphs[(id(state), bs, psize)] = (graph, out)
+                self._state_graph_lookup.clear()
                 torch.cuda.synchronize()
                 reset_context()
+
+    def _state_graph_for(self, state, rows, partition_size):
+        """The graph recorded over `state` for the smallest batch size >= rows (and the given shared-prefix
+        partition size, None = the plain launch), or None."""
+        key = (id(state), rows, partition_size)
+        hit = self._state_graph_lookup.get(key, False)
+        if hit is False:
+            sizes = sorted(bs for (sid, bs, ps) in self._state_graphs if sid == id(state) and ps == partition_size and bs >= rows)
+            hit = self._state_graphs[(id(state), sizes[0], partition_size)] if sizes else None
+            self._state_graph_lookup[key] = hit
+        return hit
 
     @torch.inference_mode()
     def run_decode_state(self, state: DecodeState) -> torch.Tensor:
@@ -755,9 +769,9 @@ class ModelRunner:
         if self.config.enable_cuda_graph:
             psize = state.prefix_partition_size if share else None
             for want in ((psize, None) if psize is not None else (None,)):
-                sizes = sorted(bs for (sid, bs, ps) in self._state_graphs if sid == id(state) and ps == want and bs >= n)
-                if sizes:
-                    graph, out = self._state_graphs[(id(state), sizes[0], want)]
+                hit = self._state_graph_for(state, n, want)
+                if hit is not None:
+                    graph, out = hit
                     graph.replay()
                     self.decode_state_stats["plain_graph" if want is None else "shared_prefix_graph"] += 1
                     return out[:n]
@@ -770,6 +784,7 @@ class ModelRunner:
     def invalidate_cuda_graphs(self):
         """Drop every recorded graph (after a weight update)."""
         self._state_graphs.clear()
+        self._state_graph_lookup.clear()
         self._prefix_groups_kept = None
         self._graphs.clear()
         self._graph_outputs.clear()

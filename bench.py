@@ -296,9 +296,29 @@ def other_decode_configs(pa, torch, dev, launches):
                                       kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
     t = time_alternating(torch, fns, launches)
+    # the merge pass of the two config-3 splits alone, inside a replayed graph (device time)
+    lib = pa._native.load()
+    merge_us = {}
+    for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3)):
+        if not psz:
+            continue
+        parts = (width3 + psz - 1) // psz
+        nbytes = lib.pa_workspace_bytes(4, HQ, D, parts)
+        ws = pa.reserve_decode_workspace(dev, nbytes)          # holds the partials of the launches timed above
+
+        def merge(ws=ws, nbytes=nbytes, psz=psz, parts=parts):
+            rc = lib.pa_merge(ws.data_ptr(), nbytes, w3["context_lens"].data_ptr(), w3["out"].data_ptr(), 0, HQ * D,
+                              4, HQ, D, psz, parts, torch.cuda.current_stream(dev).cuda_stream)
+            assert rc == 0, lib.pa_last_error()
+
+        fns[name]()                                            # partials of this split
+        torch.cuda.synchronize()
+        merge_us[name] = round(time_in_graph(torch, merge, 20, 3, reps=32) * 1e3, 2)
     for name, m in meta.items():
         us = med(t[name])
         rec = {"workload": m["workload"], "us": spread(t[name])}
+        if name in merge_us:
+            rec["merge_pass_us_in_graph"] = merge_us[name]
         if "note" in m:
             rec["note"] = m["note"]
             rec["kv_bytes"] = m["kv_bytes"]
@@ -484,7 +504,11 @@ def mfma_ceiling(pa, torch, dev):
 
 def kv_store_times(pa, torch, dev, steps, warmup):
     """Paged KV-cache write of one decode step (64 new tokens) and of one prefill chunk (4096
-    tokens), FP16 copy and FP8 quantising store.  Latency-bound: reported in microseconds only."""
+    tokens), FP16 copy and FP8 quantising store, into random slots of a pool.  Device time per call
+    inside a replayed HIP graph (16 calls per graph: eagerly a call costs its own launch, ~11 us
+    whatever it moves), and the eager time beside it.  Algorithmic bytes: K and V rows read once and
+    written once (fp8: one byte per element written, plus a 4-byte scale per token and tensor); the
+    4096-token store is bandwidth-bound and gets a GB/s figure, the 64-token one is latency-bound."""
     HKV, D, BS, NB = 8, 128, 16, 4096 // 16 + 64
     g = torch.Generator(device=dev).manual_seed(7)
     out = {}
@@ -498,9 +522,23 @@ def kv_store_times(pa, torch, dev, steps, warmup):
         v8 = torch.zeros_like(k8)
         ks = torch.ones(NB, BS, dtype=torch.float32, device=dev)
         vs = torch.ones_like(ks)
-        ms16, _ = time_steps(torch, lambda: pa.store_kv_cache(k, v, kc, vc, slots), steps, warmup)
-        ms8, _ = time_steps(torch, lambda: pa.store_kv_cache(k, v, k8, v8, slots, ks, vs, "fp8"), steps, warmup)
-        out["tokens_%d" % n] = {"fp16_us": round(ms16 * 1e3, 2), "fp8_us": round(ms8 * 1e3, 2)}
+        f16 = lambda: pa.store_kv_cache(k, v, kc, vc, slots)
+        f8 = lambda: pa.store_kv_cache(k, v, k8, v8, slots, ks, vs, "fp8")
+        ms16, _ = time_steps(torch, f16, steps, warmup)
+        ms8, _ = time_steps(torch, f8, steps, warmup)
+        g16 = time_in_graph(torch, f16, max(steps // 4, 10), 3)
+        g8 = time_in_graph(torch, f8, max(steps // 4, 10), 3)
+        bytes16 = 2 * n * HKV * D * (2 + 2)
+        bytes8 = 2 * n * (HKV * D * (2 + 1) + 4)
+        rec = {"fp16_us": round(g16 * 1e3, 2), "fp8_us": round(g8 * 1e3, 2),
+               "fp16_eager_us": round(ms16 * 1e3, 2), "fp8_eager_us": round(ms8 * 1e3, 2),
+               "fp16_algorithmic_bytes": bytes16, "fp8_algorithmic_bytes": bytes8}
+        if n == 4096:
+            rec["fp16_gbps"] = round(bytes16 / g16 / 1e6, 1)
+            rec["fp8_gbps"] = round(bytes8 / g8 / 1e6, 1)
+            rec["fp16_frac_of_8TBps"] = round(bytes16 / g16 / 1e6 / HBM_PEAK_GBPS, 4)
+            rec["fp8_frac_of_8TBps"] = round(bytes8 / g8 / 1e6 / HBM_PEAK_GBPS, 4)
+        out["tokens_%d" % n] = rec
     return out
 
 
@@ -705,6 +743,84 @@ def model_step_cfg5b(pa, torch, dev, steps, warmup):
     out["kv_bytes_per_step"] = kv_bytes
     out["kv_gbps_in_graph_step"] = round(kv_bytes / out["hip_graph_ms"] / 1e6, 1)
     del pool, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def model_step_cfg4(pa, torch, dev, steps=12):
+    """Fourth benchmark configuration through the caller: 32 prompts x 8 samples in one DecodeState of 256
+    rows, the samples aliasing their prompt's 64 blocks through the cache manager
+    (allocate_for_sequence(shared_block_ids=...)), a Qwen3-0.6B-shaped model (28 layers, random weights),
+    FP16 KV.  One step = advance kernel + replayed graph + greedy sampling on the device.  The state keeps
+    the groups of rows that share a prefix (found once, when the rows are admitted); the runner replays
+    the graph recorded over the shared-prefix launch, and - with share_prefix_decode off - the plain one.
+    Host time per step is what the Python side of a step costs (DecodeState.step + run_decode_state)."""
+    import time as _time
+    cfg = pa.Qwen3PagedConfig()
+    BS, PROMPTS, SAMPLES, PREFIX = 16, 32, 8, 1024
+    suf = _uniform_lens(torch, 1004, PROMPTS * SAMPLES, 64, 512)
+    lens = [PREFIX + x for x in suf]
+    spare = 2                                                # blocks per row for the tokens of the timed steps
+    nb = PROMPTS * (PREFIX // BS) + sum((x + BS - 1) // BS + 1 + spare for x in suf) + 64
+    torch.manual_seed(11)
+    with torch.device(dev):
+        model = pa.Qwen3PagedModel(cfg).half().eval()
+    pool = pa.BlockPool(nb, BS, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim, dtype=torch.float16, device=dev)
+    pool.kv_cache_tensor.normal_()
+    mgr = pa.KVCacheManager(pool, BS)
+    width = (max(lens) + BS - 1) // BS + spare
+    out = {"workload": "Qwen3-0.6B shape, 28 layers, 32 prompts x 8 samples (256 rows) sharing 1024-token prefixes, "
+                       "suffix U[64,512] (seed 1004), FP16 KV, one decode step"}
+    runner = pa.ModelRunner(model, pa.ModelRunnerConfig(
+        num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads, head_dim=cfg.head_dim,
+        hidden_size=cfg.hidden_size, block_size=BS, max_num_blocks=width, device="cuda:0", enable_cuda_graph=True,
+        max_cuda_graph_batch_size=PROMPTS * SAMPLES))
+    runner.bind_kv_cache(pool.kv_cache_tensor)
+    state = pa.DecodeState(PROMPTS * SAMPLES, width, BS, nb, device=dev, num_q_heads=cfg.num_heads,
+                           num_kv_heads=cfg.num_kv_heads, prefix_partition_sizes=runner.config.prefix_partition_sizes)
+    t0 = _time.perf_counter()
+    for p_ in range(PROMPTS):
+        shared = None
+        for s_ in range(SAMPLES):
+            i = p_ * SAMPLES + s_
+            table = mgr.allocate_for_sequence(i, lens[i] + spare * BS, shared_block_ids=shared).get_physical_block_ids()
+            if shared is None:
+                shared = table[:PREFIX // BS]                # the prompt's blocks: full, so the samples may alias them
+            state.admit(table, lens[i], 1)
+    state.sync_prefix_groups()
+    out["admit_256_rows_and_find_groups_host_ms"] = round((_time.perf_counter() - t0) * 1e3, 2)
+    assert state.prefix_groups_host == [(list(range(8 * i, 8 * i + 8)), PREFIX) for i in range(PROMPTS)]
+    out["prefix_partition_size"] = state.prefix_partition_size
+    runner.capture_decode_state_graphs(state, [PROMPTS * SAMPLES])
+    nxt = [None]
+    for label, share in (("shared_prefix_graph", True), ("plain_graph", False)):
+        runner.config.share_prefix_decode = share
+        before = dict(runner.decode_state_stats)
+        for _ in range(2):
+            state.step(None, nxt[0])
+            nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
+        torch.cuda.synchronize()
+        t0 = _time.perf_counter()
+        host_step = host_run = 0.0
+        for _ in range(steps):
+            h0 = _time.perf_counter()
+            state.step(None, nxt[0])
+            h1 = _time.perf_counter()
+            logits = runner.run_decode_state(state)
+            h2 = _time.perf_counter()
+            host_step += h1 - h0
+            host_run += h2 - h1
+            nxt[0] = pa.sample_tokens(logits, temperature=0.0)
+        torch.cuda.synchronize()
+        out[label + "_step_ms"] = round((_time.perf_counter() - t0) * 1e3 / steps, 3)
+        # metadata (groups included: nothing to do in a step) / picking and launching the recorded graph
+        out[label + "_host_us_per_step"] = {"DecodeState.step": round(host_step * 1e6 / steps, 1),
+                                            "run_decode_state (graph launch call)": round(host_run * 1e6 / steps, 1)}
+        taken = {k: runner.decode_state_stats[k] - before[k] for k in before}
+        assert taken[label] == steps + 2 and sum(taken.values()) == steps + 2, taken
+    out["attention_us_saved_per_step"] = round((out["plain_graph_step_ms"] - out["shared_prefix_graph_step_ms"]) * 1e3, 1)
+    runner.invalidate_cuda_graphs()
+    del pool, model, state
     torch.cuda.empty_cache()
     return out
 
@@ -977,6 +1093,7 @@ def main():
         line["block_elementwise"] = block_elementwise_times(pa, torch, dev, args.steps, args.warmup)
         line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
         line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
+        line["model_decode_step_cfg4"] = model_step_cfg4(pa, torch, dev)
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
