@@ -20,6 +20,7 @@ from .attention import (
     qk_norm_rope_store,
     sample_tokens,
     slot_mapping,
+    prefill_metadata,
     gather_kv_cache,
     add_rms_norm,
     silu_mul,
@@ -47,7 +48,7 @@ from . import _native
 
 __all__ = [
     "InferenceContext", "set_context", "get_context", "reset_context",
-    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "DecodeState", "slot_mapping", "gather_kv_cache", "add_rms_norm", "silu_mul", "HAS_FP8",
+    "Block", "BlockPool", "BlockTable", "KVCacheManager", "PrefixCache", "CachedBlock", "RadixAttentionCache", "RadixNode", "CUDAGraphRunner", "DecodeState", "slot_mapping", "prefill_metadata", "gather_kv_cache", "add_rms_norm", "silu_mul", "HAS_FP8",
     "PagedAttention", "PartitionedPagedAttention", "store_kv_cache", "qk_norm_rope_store", "sample_tokens",
     "paged_decode", "paged_decode_shared_prefix", "find_prefix_groups", "find_prefix_groups_anywhere", "PrefixGroups", "shared_prefix_descriptors", "prepare_prefix_groups", "paged_prefill", "choose_partition", "choose_launch", "reserve_decode_workspace", "sizing_graph_workspace",
     "decode_workspace_bytes", "release_decode_workspaces", "check_block_tables",

@@ -61,6 +61,7 @@ SIGNATURES = {
     "pa_silu_mul": (_int, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _int, _i64, _i64, _ptr]),
     "pa_gather_kv": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64, _ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_decode_advance": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _ptr]),
+    "pa_prefill_metadata": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_slot_mapping": (_int, [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i64, _ptr]),
     "pa_check_tables": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
 }

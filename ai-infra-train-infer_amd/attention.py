@@ -391,6 +391,44 @@ def slot_mapping(positions, block_tables, block_size, num_blocks, cu_seqlens_q=N
     return out
 
 
+def prefill_metadata(cu_seqlens_q, cu_seqlens_k, num_tokens, block_tables=None, block_size=16, num_blocks=None,
+                     row_index=None):
+    """(positions int64 [num_tokens], slot_mapping int32 [num_tokens] or None) of a prefill step,
+    computed on the GPU from its cumulative length arrays (src/inference/model_runner.py:479-511):
+    token t of chunk r sits at position cached_r + t - cu_seqlens_q[r], and its slot comes from the
+    sequence's row of block_tables (row_index[r] of a larger device-resident table when given, else
+    row r).  Without block_tables only the positions are made."""
+    _require_gpu(cu_seqlens_q, "prefill_metadata")
+    lib = _native.load()
+    cu_q = _int32(cu_seqlens_q, "prefill_metadata")
+    cu_k = _int32(cu_seqlens_k, "prefill_metadata")
+    num_seqs = cu_q.numel() - 1
+    if cu_k.numel() != num_seqs + 1:
+        raise RuntimeError("prefill_metadata: cu_seqlens_q and cu_seqlens_k differ in length")
+    positions = torch.empty(int(num_tokens), dtype=torch.long, device=cu_q.device)
+    slots = None
+    bt_ptr, bt_stride, rows, width, idx_ptr = None, 0, 0, 0, None
+    if block_tables is not None:
+        if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or block_tables.stride(1) != 1:
+            raise RuntimeError("prefill_metadata: block_tables must be int32 [rows, max_blocks] with unit column stride")
+        if num_blocks is None:
+            raise RuntimeError("prefill_metadata: num_blocks is needed with block_tables")
+        slots = torch.empty(int(num_tokens), dtype=torch.int32, device=cu_q.device)
+        bt_ptr, bt_stride, rows, width = block_tables.data_ptr(), block_tables.stride(0), block_tables.shape[0], block_tables.shape[1]
+        if row_index is not None:
+            row_index = _int32(row_index, "prefill_metadata")
+            if row_index.numel() != num_seqs:
+                raise RuntimeError("prefill_metadata: row_index must have one entry per sequence")
+            idx_ptr = row_index.data_ptr()
+        elif rows < num_seqs:
+            raise RuntimeError("prefill_metadata: block_tables has %d rows for %d sequences" % (rows, num_seqs))
+    rc = lib.pa_prefill_metadata(cu_q.data_ptr(), cu_k.data_ptr(), bt_ptr, bt_stride, idx_ptr, positions.data_ptr(),
+                                 slots.data_ptr() if slots is not None else None, int(num_tokens), num_seqs, rows, width,
+                                 int(block_size), int(num_blocks or 1), _stream_ptr(cu_q.device))
+    _native.check(rc, "pa_prefill_metadata")
+    return positions, slots
+
+
 def _device_index(device):
     return device.index if device.index is not None else torch.cuda.current_device()
 

@@ -44,6 +44,46 @@ __global__ __launch_bounds__(256) void slot_mapping_kernel(const int64_t* __rest
   slots[t] = slot;
 }
 
+// Positions and slots of the tokens of a prefill step from its two cumulative length arrays: token t
+// belongs to the sequence r whose chunk [cu_q[r], cu_q[r+1]) holds it, the sequence has
+// (cu_k[r+1] - cu_k[r]) - (cu_q[r+1] - cu_q[r]) tokens in the cache already, so the token's position
+// is that count plus its index in the chunk, and its slot follows from the sequence's table row
+// (row_index[r] of the table when given, else r).  One thread per token.
+__global__ __launch_bounds__(256) void prefill_metadata_kernel(const int32_t* __restrict__ cu_seqlens_q,
+                                                               const int32_t* __restrict__ cu_seqlens_k,
+                                                               const int32_t* __restrict__ block_tables,
+                                                               int64_t bt_stride, const int32_t* __restrict__ row_index,
+                                                               int64_t* __restrict__ positions,
+                                                               int32_t* __restrict__ slots, int64_t num_tokens,
+                                                               int num_seqs, int table_rows, int table_width,
+                                                               int block_size, int num_blocks) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= num_tokens) return;
+  if (t >= (int64_t)cu_seqlens_q[num_seqs]) {      // padding behind the last chunk
+    positions[t] = 0;
+    if (slots) slots[t] = -1;
+    return;
+  }
+  int lo = 0, hi = num_seqs;                       // last sequence whose first token is <= t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)cu_seqlens_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int r = lo;
+  const int q0 = cu_seqlens_q[r];
+  const int cached = (cu_seqlens_k[r + 1] - cu_seqlens_k[r]) - (cu_seqlens_q[r + 1] - q0);
+  const int64_t pos = (int64_t)cached + (t - q0);
+  positions[t] = pos;
+  if (!slots) return;
+  int32_t slot = -1;
+  const int row = row_index ? row_index[r] : r;
+  if (pos >= 0 && pos / block_size < table_width && row >= 0 && row < table_rows) {
+    const int32_t block = block_tables[(int64_t)row * bt_stride + pos / block_size];
+    if (block >= 0 && block < num_blocks) slot = block * block_size + (int32_t)(pos % block_size);
+  }
+  slots[t] = slot;
+}
+
 // One decode step of a batch whose metadata lives on the device: every active row (context
 // length > 0) gets one token longer, a row whose new token opens a block receives that block's id
 // from new_blocks, and position and slot of the new token follow from the row's own table.  One
@@ -105,6 +145,27 @@ extern "C" int pa_slot_mapping(const int64_t* positions, const int32_t* cu_seqle
                      cu_seqlens_q, block_tables, bt_stride, slots, num_tokens, (int)num_rows, (int)table_width,
                      (int)block_size, (int)num_blocks);
   return check_launch("pa_slot_mapping");
+}
+
+extern "C" int pa_prefill_metadata(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* block_tables,
+                                   int64_t bt_stride, const int32_t* row_index, int64_t* positions, int32_t* slots,
+                                   int64_t num_tokens, int64_t num_seqs, int64_t table_rows, int64_t table_width,
+                                   int64_t block_size, int64_t num_blocks, void* stream) {
+  if (num_tokens < 0 || num_seqs < 0 || table_rows < 0 || table_width < 0 || block_size <= 0 || num_blocks <= 0)
+    return fail(PA_ERR_BAD_ARG, "pa_prefill_metadata: negative or zero size");
+  if (num_tokens == 0) return PA_OK;
+  if (!cu_seqlens_q || !cu_seqlens_k || !positions) return fail(PA_ERR_BAD_ARG, "pa_prefill_metadata: null pointer");
+  if (num_seqs == 0) return fail(PA_ERR_BAD_ARG, "pa_prefill_metadata: tokens but no sequences");
+  if (slots && !block_tables) return fail(PA_ERR_BAD_ARG, "pa_prefill_metadata: slots need block tables");
+  if (slots && bt_stride < table_width) return fail(PA_ERR_BAD_ARG, "pa_prefill_metadata: table stride smaller than its width");
+  if (num_seqs > INT32_MAX || table_rows > INT32_MAX || table_width > INT32_MAX || num_blocks * block_size > INT32_MAX)
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill_metadata: slots must fit int32");
+  const int64_t wgs = (num_tokens + 255) / 256;
+  if (wgs > INT32_MAX) return fail(PA_ERR_UNSUPPORTED, "pa_prefill_metadata: too many tokens for one launch");
+  hipLaunchKernelGGL(prefill_metadata_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, cu_seqlens_q,
+                     cu_seqlens_k, block_tables, bt_stride, row_index, positions, slots, num_tokens, (int)num_seqs,
+                     (int)table_rows, (int)table_width, (int)block_size, (int)num_blocks);
+  return check_launch("pa_prefill_metadata");
 }
 
 extern "C" int pa_decode_advance(int32_t* block_tables, int64_t bt_stride, int32_t* context_lens, int64_t* positions,

@@ -255,6 +255,51 @@ class KVCacheManager:
         self._block_size = block_size
         self._seq_tables: Dict[object, BlockTable] = {}
         self._pending_copies: List[Tuple[int, int]] = []
+        # Which sequences may share a prefix, recorded where sharing is made (a prefix-cache hit, a fork)
+        # and dropped where it ends (free, a private copy of the first block): sequences that share
+        # anything share their first physical block, so the index is first block id -> sequences.
+        self._by_first_block: Dict[int, Set[object]] = {}
+        self._first_block_of: Dict[object, int] = {}
+
+    # -- who shares with whom -----------------------------------------------------------------
+
+    def _index_first_block(self, seq_id):
+        """Keep the first-block index in step with the sequence's table."""
+        table = self._seq_tables.get(seq_id)
+        new = table.blocks[0].block_id if table is not None and table.blocks else None
+        old = self._first_block_of.get(seq_id)
+        if new == old:
+            return
+        if old is not None:
+            members = self._by_first_block.get(old)
+            if members is not None:
+                members.discard(seq_id)
+                if not members:
+                    del self._by_first_block[old]
+            del self._first_block_of[seq_id]
+        if new is not None:
+            self._by_first_block.setdefault(new, set()).add(seq_id)
+            self._first_block_of[seq_id] = new
+
+    def sharing_candidates(self) -> List[List[object]]:
+        """Sets of live sequences that start with the same physical block, i.e. that share a prefix
+        (only sets of two or more)."""
+        return [sorted(m, key=repr) for m in self._by_first_block.values() if len(m) > 1]
+
+    def shared_prefix_groups(self, seq_ids, num_q_heads: int, num_kv_heads: int, partition_size: int):
+        """Groups of the given sequences that share a prefix of whole partitions, as
+        [([index into seq_ids, ...], shared_tokens)] - what attention.shared_prefix_descriptors takes for a
+        batch whose rows are seq_ids.  Only sequences the index names as sharers are looked at: a batch
+        without sharing costs one dictionary lookup per row."""
+        from .attention import find_prefix_groups_anywhere
+        rows = [i for i, s in enumerate(seq_ids)
+                if len(self._by_first_block.get(self._first_block_of.get(s, -1), ())) > 1]
+        if len(rows) < 2:
+            return []
+        tables = [self._seq_tables[seq_ids[i]].get_physical_block_ids() for i in rows]
+        lens = [self._seq_tables[seq_ids[i]].num_tokens for i in rows]
+        return find_prefix_groups_anywhere(tables, lens, self._block_size, num_q_heads, num_kv_heads, partition_size,
+                                           rows=rows)
 
     # -- allocation ---------------------------------------------------------------------------
 
@@ -291,6 +336,7 @@ class KVCacheManager:
             block.is_full = block.token_count == self._block_size
             table.append_block(block)
         self._seq_tables[seq_id] = table
+        self._index_first_block(seq_id)
         return table
 
     def fork_sequence(self, parent_id, child_id) -> BlockTable:
@@ -306,6 +352,7 @@ class KVCacheManager:
             table.append_block(self._pool.share(block))
         table._last_tokens = parent._last_tokens
         self._seq_tables[child_id] = table
+        self._index_first_block(child_id)
         return table
 
     def append_token(self, seq_id) -> bool:
@@ -322,6 +369,8 @@ class KVCacheManager:
             block.token_count = 1
             block.is_full = self._block_size == 1
             table.append_block(block)
+            if table.num_blocks == 1:
+                self._index_first_block(seq_id)
             return True
         if last.ref_count > 1:
             block = self._pool.allocate()
@@ -333,6 +382,8 @@ class KVCacheManager:
             block.is_full = block.token_count == self._block_size
             table._blocks[-1] = block
             table._last_tokens = block.token_count
+            if table.num_blocks == 1:
+                self._index_first_block(seq_id)           # the private copy is the sequence's first block now
             return True
         last.token_count = table._last_tokens + 1
         last.is_full = last.token_count == self._block_size
@@ -376,6 +427,7 @@ class KVCacheManager:
         table = self._seq_tables.pop(seq_id, None)
         if table is None:
             return
+        self._index_first_block(seq_id)
         for block in table.blocks:
             self._pool.free(block)
 

@@ -139,7 +139,7 @@ class DecodeState:
             raise RuntimeError("DecodeState.admit: a sequence enters decode with at least one cached token")
         if len(block_table) > self.max_blocks or len(block_table) * self.block_size < num_cached_tokens:
             raise RuntimeError("DecodeState.admit: block table does not fit the state or the tokens")
-        free = np.flatnonzero(self._lens == 0)
+        free = np.flatnonzero((self._lens == 0) & (self._ntab == 0))
         if not free.size:
             raise RuntimeError("DecodeState.admit: all %d rows are in use" % self.max_batch)
         row = int(free[0])
@@ -155,6 +155,37 @@ class DecodeState:
         self._ntab[row] = len(block_table)
         self._groups_dirty = self.tracks_prefixes
         return row
+
+    def reserve(self, block_table: List[int]) -> int:
+        """Give a sequence that has not finished its prefill the lowest free row: its block table goes to
+        the device now (prefill chunks can take it from there: ModelRunner.prepare_prefill(state=...)), the
+        row stays out of the decode steps until activate().  Returns the row."""
+        if not block_table or len(block_table) > self.max_blocks:
+            raise RuntimeError("DecodeState.reserve: block table empty or wider than the state")
+        free = np.flatnonzero((self._lens == 0) & (self._ntab == 0))
+        if not free.size:
+            raise RuntimeError("DecodeState.reserve: all %d rows are in use" % self.max_batch)
+        row = int(free[0])
+        host_row = torch.full((self.max_blocks,), -1, dtype=torch.int32)
+        host_row[:len(block_table)] = torch.tensor(block_table, dtype=torch.int32)
+        self.block_tables[row].copy_(host_row.pin_memory(), non_blocking=True)
+        self._tables[row] = list(block_table)
+        self._ntab[row] = len(block_table)
+        return row
+
+    def activate(self, row: int, num_cached_tokens: int, next_token: int):
+        """A reserved row joins the decode steps: its `num_cached_tokens` tokens are in the cache and
+        `next_token` is the one its last prefill chunk produced."""
+        if self._lens[row] != 0 or self._ntab[row] == 0:
+            raise RuntimeError("DecodeState.activate: row %d is not a reserved row" % row)
+        if num_cached_tokens <= 0 or self._ntab[row] * self.block_size < num_cached_tokens:
+            raise RuntimeError("DecodeState.activate: the row's block table does not hold %d tokens" % num_cached_tokens)
+        self.context_lens[row].fill_(int(num_cached_tokens))
+        self.input_ids[row].fill_(int(next_token))
+        self._fresh[row].fill_(1)
+        self._fresh_rows.add(row)
+        self._lens[row] = int(num_cached_tokens)
+        self._groups_dirty = self.tracks_prefixes
 
     def retire(self, row: int) -> List[int]:
         """Free a row; returns the block ids the sequence held."""
@@ -382,9 +413,79 @@ class ModelRunner:
                 tables[i, :len(bt)] = bt
         return self._to_device(tables, torch.int32)
 
-    def prepare_prefill(self, sequences: List[dict]) -> Tuple[torch.Tensor, torch.Tensor]:
+    def prepare_prefill(self, sequences: List[dict], state: Optional["DecodeState"] = None
+                        ) -> Tuple[torch.Tensor, torch.Tensor]:
         """sequences: dicts with 'token_ids', 'block_table', 'num_cached_tokens',
-        'num_scheduled_tokens'.  Sets the global context; returns (input_ids, positions)."""
+        'num_scheduled_tokens'.  Sets the global context; returns (input_ids, positions).
+
+        On the GPU the step's metadata goes up in ONE copy - the chunk's token ids, the two cumulative
+        length arrays and (when a sequence has a cached prefix or a cache to write) the block tables,
+        side by side in one pinned buffer - and positions and slots are computed there by
+        pa_prefill_metadata; the reference builds them in Python loops and ships every field on its own
+        (src/inference/model_runner.py:464-540).  With `state` and a 'state_row' in every dict (a row
+        the sequence holds in the DecodeState: DecodeState.reserve) the tables are not sent at all:
+        they are the state's own rows, which stay on the device from the first chunk to the last
+        decode step."""
+        if self._device() == "cpu":
+            return self._prepare_prefill_host(sequences)
+        from .attention import prefill_metadata
+        dev = torch.device(self._device())
+        S = len(sequences)
+        starts = [seq["num_cached_tokens"] for seq in sequences]
+        counts = [seq["num_scheduled_tokens"] for seq in sequences]
+        total = sum(counts)
+        from_state = state is not None and S > 0 and all("state_row" in seq for seq in sequences)
+        lists = [seq.get("block_table", []) for seq in sequences]
+        any_table = any(len(bt) for bt in lists)
+        has_prefix = any(st > 0 for st in starts)
+        width = 0 if from_state or not any_table else max(len(bt) for bt in lists)
+        # one pinned staging buffer: ids int64 [total] | cu_q int32 [S+1] | cu_k int32 [S+1] | rows int32 [S] | tables int32 [S, width]
+        n32 = 2 * (S + 1) + S + S * width
+        stage = torch.empty(8 * total + 4 * n32, dtype=torch.uint8).pin_memory()
+        ids = stage[:8 * total].view(torch.long)
+        meta = stage[8 * total:].view(torch.int32)
+        ids_np, meta_np = ids.numpy(), meta.numpy()
+        cu_q, cu_k = meta_np[:S + 1], meta_np[S + 1:2 * (S + 1)]
+        rows_np = meta_np[2 * (S + 1):2 * (S + 1) + S]
+        tables_np = meta_np[2 * (S + 1) + S:].reshape(S, width) if width else None
+        cu_q[0] = cu_k[0] = 0
+        cursor = max_q = max_k = 0
+        if tables_np is not None:
+            tables_np.fill(-1)
+        for i, seq in enumerate(sequences):
+            start, n = starts[i], counts[i]
+            ids_np[cursor:cursor + n] = seq["token_ids"][start:start + n]
+            cursor += n
+            cu_q[i + 1] = cu_q[i] + n
+            cu_k[i + 1] = cu_k[i] + start + n
+            max_q, max_k = max(max_q, n), max(max_k, start + n)
+            rows_np[i] = seq["state_row"] if from_state else i
+            if tables_np is not None and len(lists[i]):
+                tables_np[i, :len(lists[i])] = lists[i]
+        on_dev = stage.to(dev, non_blocking=True)
+        input_ids = on_dev[:8 * total].view(torch.long)
+        meta_dev = on_dev[8 * total:].view(torch.int32)
+        cu_q_dev, cu_k_dev = meta_dev[:S + 1], meta_dev[S + 1:2 * (S + 1)]
+        rows_dev = meta_dev[2 * (S + 1):2 * (S + 1) + S]
+        num_blocks = self._kv_cache.shape[2] if self._kv_cache is not None else 2 ** 31 // self.block_size - 1
+        if from_state:
+            positions, slot_mapping = prefill_metadata(cu_q_dev, cu_k_dev, total, state.block_tables, self.block_size,
+                                                       num_blocks, row_index=rows_dev)
+            block_tables = state.block_tables.index_select(0, rows_dev.long()) if has_prefix else None
+        elif width:
+            tables_dev = meta_dev[2 * (S + 1) + S:].view(S, width)
+            positions, slot_mapping = prefill_metadata(cu_q_dev, cu_k_dev, total, tables_dev, self.block_size, num_blocks)
+            block_tables = tables_dev if has_prefix else None
+        else:
+            positions, slot_mapping = prefill_metadata(cu_q_dev, cu_k_dev, total)
+            block_tables = None
+        set_context(is_prefill=True, cu_seqlens_q=cu_q_dev, cu_seqlens_k=cu_k_dev, max_seqlen_q=max_q, max_seqlen_k=max_k,
+                    slot_mapping=slot_mapping, block_tables=block_tables)
+        return input_ids, positions
+
+    def _prepare_prefill_host(self, sequences: List[dict]) -> Tuple[torch.Tensor, torch.Tensor]:
+        """prepare_prefill with every field built on the host (numpy row copies): what a machine without
+        a GPU runs, and what the device path is checked against."""
         ids, pos, slots = [], [], []
         cu_q, cu_k = [0], [0]
         max_q = max_k = 0

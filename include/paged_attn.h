@@ -409,6 +409,23 @@ int pa_silu_mul(const void* gate, int64_t gate_stride, const void* up, int64_t u
                 int64_t out_stride, int dtype, int64_t rows, int64_t width, void* stream);
 
 /*
+ * Positions and cache slots of the tokens of one prefill step, on the device, from the step's two
+ * cumulative length arrays (int32 [num_seqs + 1]: new tokens, and cached + new tokens, per sequence):
+ * token t of chunk r gets positions[t] = cached_r + (t - cu_seqlens_q[r]) (int64) and
+ * slots[t] = block_tables[row][positions[t] / block_size] * block_size + positions[t] % block_size
+ * with row = row_index[r] (optional int32 [num_seqs]: the sequences' rows in a larger, device-resident
+ * table of table_rows rows) or r.  slots may be NULL (no cache bound).  Tokens at or past
+ * cu_seqlens_q[num_seqs] get position 0 and slot -1; a position past the table, a row outside it or
+ * a block id outside [0, num_blocks) gives slot -1, which the KV writers skip.
+ * Replaces: the position and slot loops of ModelRunner.prepare_prefill
+ * (src/inference/model_runner.py:479-511) and the two uploads they end in.
+ */
+int pa_prefill_metadata(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* block_tables,
+                        int64_t bt_stride, const int32_t* row_index, int64_t* positions, int32_t* slots,
+                        int64_t num_tokens, int64_t num_seqs, int64_t table_rows, int64_t table_width,
+                        int64_t block_size, int64_t num_blocks, void* stream);
+
+/*
  * slots[t] = block_tables[row(t)][positions[t] / block_size] * block_size + positions[t] % block_size
  * for num_tokens tokens, all on the device.  cu_seqlens_q == NULL: token t belongs to table row t
  * (one new token per sequence, num_tokens == num_rows).  Otherwise cu_seqlens_q is int32

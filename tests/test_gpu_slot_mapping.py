@@ -176,3 +176,93 @@ def test_graph_runner_replays_equal_eager_and_padding_rows_are_inert(pa, gpu):
     runner.invalidate()
     assert not runner.is_captured(2) and runner.get_stats()["captured_sizes"] == []
     pa.reset_context()
+
+
+def test_prepare_prefill_on_the_device_equals_the_reference_loops(pa, gpu):
+    """ModelRunner.prepare_prefill on the GPU: one upload (ids, cumulative lengths, tables), positions and
+    slots made by pa_prefill_metadata - every field equal to the reference's host loops."""
+    import random
+    from test_model_runner_host import random_sequences, as_list
+    rng = random.Random(12)
+    for bs in (8, 16):
+        runner = pa.ModelRunner(None, pa.ModelRunnerConfig(block_size=bs, device="cuda:0"))
+        for trial in range(6):
+            seqs = random_sequences(rng, rng.randint(1, 9), bs, prefill=True)
+            if trial == 5:
+                for s in seqs:
+                    s["num_cached_tokens"] = 0                         # no prefix anywhere: no tables in the context
+                    s["num_scheduled_tokens"] = min(s["num_scheduled_tokens"], len(s["block_table"]) * bs)
+            ids, pos = runner.prepare_prefill(seqs)
+            ctx = pa.get_context()
+            torch.cuda.synchronize()
+            want = mro.prefill_metadata(seqs, bs)
+            assert ids.is_cuda and ids.dtype == torch.long and pos.dtype == torch.long
+            assert ids.tolist() == want["input_ids"] and pos.tolist() == want["positions"]
+            assert ctx.is_prefill and as_list(ctx.slot_mapping) == want["slot_mapping"]
+            assert as_list(ctx.cu_seqlens_q) == want["cu_seqlens_q"] and as_list(ctx.cu_seqlens_k) == want["cu_seqlens_k"]
+            assert (ctx.max_seqlen_q, ctx.max_seqlen_k) == (want["max_seqlen_q"], want["max_seqlen_k"])
+            assert as_list(ctx.block_tables) == want["block_tables"]
+            for t in (ctx.slot_mapping, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.block_tables):
+                assert t is None or (t.dtype == torch.int32 and t.is_cuda)
+    # no tables at all: positions only
+    runner.prepare_prefill([{"token_ids": [1, 2, 3], "num_cached_tokens": 0, "num_scheduled_tokens": 3}])
+    ctx = pa.get_context()
+    assert ctx.slot_mapping is None and ctx.block_tables is None
+    pa.reset_context()
+
+
+def test_prefill_chunks_take_their_tables_from_the_decode_state(pa, gpu):
+    """Sequences reserve a DecodeState row before their first chunk: the block table goes to the device
+    once, every chunk's slots come from that row, and the row joins the decode steps when the prompt is in."""
+    bs, NB = 16, 400
+    g = torch.Generator().manual_seed(43)
+    free = torch.randperm(NB, generator=g).tolist()
+    st = pa.DecodeState(6, 16, bs, NB, device=gpu)
+    runner = pa.ModelRunner(None, pa.ModelRunnerConfig(block_size=bs, device="cuda:0"))
+    st.admit([free.pop()], 5, 9)                                   # row 0 is taken by a decoding sequence
+    seqs = []
+    for total in (150, 40, 97):
+        table = [free.pop() for _ in range((total + bs - 1) // bs)]
+        row = st.reserve(table)
+        seqs.append({"token_ids": [int(x) for x in torch.randint(0, 999, (total,), generator=g)], "block_table": table,
+                     "state_row": row, "num_cached_tokens": 0, "num_scheduled_tokens": 0})
+    assert [s["state_row"] for s in seqs] == [1, 2, 3] and st.rows_in_use == 1      # reserved rows do not decode yet
+    chunk = 64
+    while any(s["num_cached_tokens"] < len(s["token_ids"]) for s in seqs):
+        batch = []
+        for s in seqs:
+            left = len(s["token_ids"]) - s["num_cached_tokens"]
+            if left:
+                s["num_scheduled_tokens"] = min(chunk, left)
+                batch.append(s)
+        ids, pos = runner.prepare_prefill(batch, state=st)
+        ctx = pa.get_context()
+        torch.cuda.synchronize()
+        want = mro.prefill_metadata(batch, bs)
+        assert ids.tolist() == want["input_ids"] and pos.tolist() == want["positions"]
+        assert ctx.slot_mapping.tolist() == want["slot_mapping"]
+        assert ctx.cu_seqlens_q.tolist() == want["cu_seqlens_q"] and ctx.cu_seqlens_k.tolist() == want["cu_seqlens_k"]
+        if want["block_tables"] is None:
+            assert ctx.block_tables is None
+        else:                                                     # the state's rows: wider than the reference's, same entries
+            got = ctx.block_tables.tolist()
+            for g_row, w_row in zip(got, want["block_tables"]):
+                real = [x for x in w_row if x >= 0]
+                assert g_row[:len(real)] == real and all(x == -1 for x in g_row[len(real):])
+        for s in batch:
+            s["num_cached_tokens"] += s["num_scheduled_tokens"]
+    for s in seqs:
+        st.activate(s["state_row"], len(s["token_ids"]), 7)
+    assert st.rows_in_use == 4
+    st.step(None)
+    torch.cuda.synchronize()
+    assert st.context_lens.tolist()[:4] == [6, 151, 41, 98]
+    want_slots = [s["block_table"][len(s["token_ids"]) // bs] * bs + len(s["token_ids"]) % bs if len(s["token_ids"]) % bs
+                  else -1 for s in seqs]
+    got_slots = st.slot_mapping.tolist()[1:4]
+    for s, got_s, want_s in zip(seqs, got_slots, want_slots):
+        if len(s["token_ids"]) % bs:
+            assert got_s == want_s
+    with pytest.raises(RuntimeError, match="not a reserved row"):
+        st.activate(1, 10, 3)
+    pa.reset_context()

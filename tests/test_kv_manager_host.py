@@ -252,3 +252,33 @@ def test_prefix_cache_eviction_order():
     assert c.match_prefix([50]) == (1, [4])
     c.insert([60], [5])
     assert c.size == 3 and c.match_prefix([10])[0] == 0 and c.get_stats()["evictions"] == 3
+
+
+def test_manager_records_who_shares_a_prefix():
+    """The first-block index follows allocation with shared blocks, forks, the private copy of a shared
+    first block and frees; shared_prefix_groups answers from it without walking unrelated tables."""
+    p = pool(64)
+    m = pa.KVCacheManager(p, BS)
+    a = m.allocate_for_sequence("a", 4 * BS + 1).get_physical_block_ids()          # 4 full blocks + 1 token
+    assert m.sharing_candidates() == []
+    m.allocate_for_sequence("b", 4 * BS + 2, shared_block_ids=a[:4])                 # a prefix-cache hit on a's 4 full blocks
+    m.allocate_for_sequence("c", 3 * BS)                                            # shares nothing
+    m.fork_sequence("a", "a2")
+    assert m.sharing_candidates() == [["a", "a2", "b"]]
+    # the batch's rows in any order; heads 2 / 1: up to 8 rows per group; partitions of two blocks
+    groups = m.shared_prefix_groups(["c", "b", "a", "a2"], 2, 1, 2 * BS)
+    assert groups == [([1, 2, 3], 4 * BS)]
+    assert m.shared_prefix_groups(["c", "a"], 2, 1, 2 * BS) == []                   # a's sharers are not in this batch
+    assert m.shared_prefix_groups(["c", "b", "a"], 32, 1, 2 * BS) == []             # no room for a second row per group
+    # a sequence whose only block is shared gets a private first block when it appends: it leaves its set
+    m.allocate_for_sequence("s", 2)
+    m.fork_sequence("s", "s2")
+    assert sorted(map(tuple, m.sharing_candidates())) == [("a", "a2", "b"), ("s", "s2")]
+    assert m.append_token("s2")
+    assert m.sharing_candidates() == [["a", "a2", "b"]]
+    m.free_sequence("b")
+    m.free_sequence("a")
+    assert m.sharing_candidates() == [] and m.shared_prefix_groups(["a2", "c"], 2, 1, 2 * BS) == []
+    for s in ("a2", "c", "s", "s2"):
+        m.free_sequence(s)
+    assert m._by_first_block == {} and m._first_block_of == {} and p.num_free_blocks == 64
