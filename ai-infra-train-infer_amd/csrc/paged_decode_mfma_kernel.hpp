@@ -15,9 +15,10 @@
 //    non-temporal unless a neighbouring row maps the same blocks.
 //  * A landed tile is written (16-bit caches as they are, bf16 and fp8 converted to fp16: K bytes of
 //    an fp8 cache as they are - exact in fp16 - with 1 / k_scale of the tile's tokens beside the tile
-//    in LDS and applied to the scores after the first product, V dequantised with 1 / v_scale on the
-//    way in) to the wave's own 2 x 32 x head_dim fp16 of LDS, and the next tile's loads are issued
-//    into the freed registers before the products start.
+//    in LDS and applied to the scores after the first product; V bytes times the power of two of
+//    1 / v_scale, exact as well, the mantissa of 1 / v_scale going into the probabilities) to the
+//    wave's own 2 x 32 x head_dim fp16 of LDS, and the next tile's loads are issued into the freed
+//    registers before the products start.
 //  * S^T = K . Q^T with v_mfma_f32_16x16x32_f16: A = 16 keys x 32 dims read back with
 //    ds_read_b128, B = Q^T (16 head columns, zero beyond the group) kept in registers, pre-scaled
 //    by scale*log2(e) and, for 16-bit caches, split into two fp16 parts (hi + lo, two products per
@@ -55,9 +56,9 @@ __device__ __forceinline__ constexpr int lds_swz(int row) {
 
 // K and V tile of one KV head
 __host__ __device__ constexpr int decode_mfma_tile_bytes(int D) { return 2 * kMfmaTile * D * 2; }
-// per wave: its tiles, then 1 / k_scale of the tile's 32 tokens (fp8 caches)
+// per wave: its tiles, then per token of the tile 1 / k_scale and the mantissa of 1 / v_scale (fp8 caches)
 __host__ __device__ constexpr int decode_mfma_wave_bytes(int HPW, int D) {
-  return HPW * decode_mfma_tile_bytes(D) + kMfmaTile * 4;
+  return HPW * decode_mfma_tile_bytes(D) + 2 * kMfmaTile * 4;
 }
 __host__ __device__ constexpr int decode_mfma_lds_bytes(int W, int HPW, int D) {
   return W * decode_mfma_wave_bytes(HPW, D) + 2 * HPW * kMfmaHeads * W * 4;
@@ -102,19 +103,14 @@ __device__ __forceinline__ mhalf8_t words_to_f16(const uint32_t* w) {
   return r;
 }
 
-// 8 fp8 bytes (2 dwords) times a per-token factor -> 8 fp16: byte * f = byte * m * 2^e with m in
-// [1, 2); v_cvt_scalef32_pk_f16_fp8 applies the power of two exactly while it converts a pair (it
-// uses only the exponent of its scale operand) and the mantissa is one packed fp16 multiply per pair.
-__device__ __forceinline__ mhalf8_t fp8_words_to_f16_scaled(const uint32_t* w, float factor) {
-  const uint32_t bits = __float_as_uint(factor);
-  const float pow2 = __uint_as_float(bits & 0xff800000u);
-  const _Float16 m = (_Float16)__uint_as_float((bits & 0x007fffffu) | 0x3f800000u);
-  const half2_t mm = {m, m};
+// 8 fp8 bytes (2 dwords) times a power of two -> 8 fp16, exactly: v_cvt_scalef32_pk_f16_fp8 applies the
+// exponent of its scale operand while it converts a pair.
+__device__ __forceinline__ mhalf8_t fp8_words_to_f16_pow2(const uint32_t* w, float pow2) {
   mhalf8_t r;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const half2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, false) * mm;
-    const half2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, true) * mm;
+    const half2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, false);
+    const half2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], pow2, true);
     r[4 * i] = lo[0];
     r[4 * i + 1] = lo[1];
     r[4 * i + 2] = hi[0];
@@ -147,7 +143,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   constexpr int WAVEB = decode_mfma_wave_bytes(HPW, D);
   uint8_t* my_lds = lds_raw + wave * WAVEB;            // this wave's tiles: per KV head K, then V
-  float* my_scales = reinterpret_cast<float*>(my_lds + HPW * TILEB);   // [TILE]: 1 / k_scale per token
+  float* my_scales = reinterpret_cast<float*>(my_lds + HPW * TILEB);   // [2][TILE]: 1 / k_scale, mantissa of 1 / v_scale per token
   float (*red)[HPW * NHC * D] = reinterpret_cast<float (*)[HPW * NHC * D]>(lds_raw);   // [W][HPW * NHC * D], over the tiles
   float (*sm)[W] = reinterpret_cast<float (*)[W]>(lds_raw + W * WAVEB);                // [HPW * NHC][W]
   float (*sl)[W] = sm + HPW * NHC;                                                      // [HPW * NHC][W]
@@ -344,12 +340,15 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     for (int r = 0; r < RL; ++r) {
       const int tk = token_of(r);
       const bool valid = !masked || (begin + tile * TILE + tk) < end;
-      // fp8: V is dequantised here, on its way into LDS (value = byte / v_scale, rounded to fp16), so
-      // that the probabilities stay pure numbers in [0, 256] when they are rounded to fp16 for the
-      // second product.  (Folding 1 / v_scale into the probability instead loses every key whose
-      // p / v_scale falls below fp16's smallest subnormal while its p still counts in the row sum.)
-      float inv_vs = 1.0f;
-      if constexpr (KV == KV_FP8) inv_vs = __builtin_amdgcn_rcpf(t.vs[r]);
+      // fp8: 1 / v_scale = m * 2^e with m in [1, 2).  The power of two goes into V here, on its way
+      // into LDS (exact, and free: the conversion instruction applies it), the mantissa into the
+      // probability before the second product, so that what is rounded to fp16 there is p * m, a number
+      // in [0, 512].  (Folding all of 1 / v_scale - about amax / 448 - into the probability loses
+      // every key whose p / v_scale falls below fp16's smallest subnormal while its p still counts in
+      // the row sum: with small V behind an attention sink, tens of percent of the output.)
+      float v_pow2 = 1.0f;
+      if constexpr (KV == KV_FP8)
+        v_pow2 = __uint_as_float(__float_as_uint(__builtin_amdgcn_rcpf(t.vs[r])) & 0xff800000u);
 #pragma unroll
       for (int c = 0; c < G::NLD; ++c) {
 #pragma unroll
@@ -358,7 +357,7 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
           const int wpc = (KV == KV_FP8) ? 2 : 4;   // dwords per 8 source elements
           mhalf8_t kf = words_to_f16<KV>(&t.k[r][c * (G::LB / 4) + x * wpc]);
           mhalf8_t vf;
-          if constexpr (KV == KV_FP8) vf = fp8_words_to_f16_scaled(&t.v[r][c * (G::LB / 4) + x * wpc], inv_vs);
+          if constexpr (KV == KV_FP8) vf = fp8_words_to_f16_pow2(&t.v[r][c * (G::LB / 4) + x * wpc], v_pow2);
           else vf = words_to_f16<KV>(&t.v[r][c * (G::LB / 4) + x * wpc]);
           if (!valid) {
             // rows past the end: their scores are masked, and their V must not turn 0 * garbage into NaN
@@ -372,18 +371,23 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       }
     }
     if constexpr (KV == KV_FP8) {
-      // 1 / k_scale per token (applied to the scores after the first product), 0 for rows past the end
-      // (their scores are masked anyway).  The 8 lanes of a row group (and both heads' groups) hold the
-      // same values and write the same words.
+      // per token: 1 / k_scale (applied to the scores after the first product) and the mantissa of
+      // 1 / v_scale (applied to the probabilities before the second); 0 for rows past the end (their
+      // scores are masked and their V rows zero, and 0 * 0 stays 0).  The 8 lanes of a row group (and
+      // both heads' groups) hold the same values and write the same words.
 #pragma unroll
       for (int sb = 0; sb < NSUB; ++sb) {
-        float ik[4];
+        float ik[4], mv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const bool valid = !masked || (begin + tile * TILE + token_of(4 * sb + r)) < end;
           ik[r] = valid ? __builtin_amdgcn_rcpf(t.ks[4 * sb + r]) : 0.0f;
+          const uint32_t bits = __float_as_uint(__builtin_amdgcn_rcpf(t.vs[4 * sb + r]));
+          mv[r] = valid ? __uint_as_float((bits & 0x007fffffu) | 0x3f800000u) : 0.0f;
         }
-        *(float4*)&my_scales[token_of(4 * sb)] = make_float4(ik[0], ik[1], ik[2], ik[3]);
+        const int tok0 = token_of(4 * sb);
+        *(float4*)&my_scales[tok0] = make_float4(ik[0], ik[1], ik[2], ik[3]);
+        *(float4*)&my_scales[TILE + tok0] = make_float4(mv[0], mv[1], mv[2], mv[3]);
       }
     }
   };
@@ -431,13 +435,15 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
         s2[hh][kb] = mfloat4_t{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
-    // fp8: 1 / k_scale of this lane's 8 keys (4kg .. 4kg+3 of both halves)
-    float iks[2][4];
+    // fp8: 1 / k_scale and the mantissa of 1 / v_scale of this lane's 8 keys (4kg .. 4kg+3 of both halves)
+    float iks[2][4], mvs[2][4];
     if constexpr (KV == KV_FP8) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         const float4 a = *(const float4*)&my_scales[16 * kb + 4 * kg];
+        const float4 b2 = *(const float4*)&my_scales[TILE + 16 * kb + 4 * kg];
         iks[kb][0] = a.x; iks[kb][1] = a.y; iks[kb][2] = a.z; iks[kb][3] = a.w;
+        mvs[kb][0] = b2.x; mvs[kb][1] = b2.y; mvs[kb][2] = b2.z; mvs[kb][3] = b2.w;
       }
     }
 #pragma unroll
@@ -504,11 +510,19 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
-          // the row sum adds exactly the fp16 values that the second product multiplies
-          const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
-          psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
-          pb[hh][4 * kb + e] = h[0];
-          pb[hh][4 * kb + e + 1] = h[1];
+          if constexpr (KV == KV_FP8) {
+            // the row sum takes the probability, the product the probability times the mantissa of 1 / v_scale
+            const float p0 = __builtin_amdgcn_exp2f(s[hh][kb][e]), p1 = __builtin_amdgcn_exp2f(s[hh][kb][e + 1]);
+            psum += p0 + p1;
+            pb[hh][4 * kb + e] = (_Float16)(p0 * mvs[kb][e]);
+            pb[hh][4 * kb + e + 1] = (_Float16)(p1 * mvs[kb][e + 1]);
+          } else {
+            // the row sum adds exactly the fp16 values that the second product multiplies
+            const half2_t h = {(_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e]), (_Float16)__builtin_amdgcn_exp2f(s[hh][kb][e + 1])};
+            psum = __builtin_amdgcn_fdot2(h, one2, psum, false);
+            pb[hh][4 * kb + e] = h[0];
+            pb[hh][4 * kb + e + 1] = h[1];
+          }
         }
       l_run[hh] += psum;
     }

@@ -97,19 +97,43 @@ def build_workload(pa, torch, dev, batch, ctx, hq, hkv, d, bs, fp8, seed):
                 block_tables=tables, context_lens=lens, num_blocks=nb)
 
 
+TRAFFIC_PROFILE = os.path.join("profiles", "paged_decode_bs64_ctx4096_pmc_traffic.txt")
+DECODE_KERNEL_SOURCES = ("paged_decode_kernel.hpp", "paged_decode_launch.hpp", "paged_decode.hip", "pa_common.hpp")
+
+
+def decode_sources_digest():
+    """sha256 over the sources of the headline's decode kernel and its launch shaping: the counter
+    summary under profiles/ records the digest it was taken at."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in DECODE_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "ai-infra-train-infer_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(key):
     """HBM bytes per launch of the decode kernel as measured with rocprofv3 --pmc FETCH_SIZE /
-    WRITE_SIZE (scaled by a plain copy of known size); read from the committed summary of those
-    runs, None if it is absent.  Counters cannot be sampled from inside this process."""
-    path = os.path.join(ROOT, "profiles", "paged_decode_bs64_ctx4096_pmc_traffic.txt")
+    WRITE_SIZE (scaled by a plain copy of known size).  Counters cannot be sampled from inside this
+    process, so the figure is read from the committed summary of those runs - and only when that
+    summary was taken at the kernel sources this run uses (it records their digest); otherwise, or
+    when the file is absent, None.  Returns (bytes or None, note)."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    value = digest = None
     try:
         with open(path) as f:
             for ln in f:
                 if ln.startswith(key + " ="):
-                    return int(ln.split("=")[1])
+                    value = int(ln.split("=")[1])
+                elif ln.startswith("decode_sources_digest ="):
+                    digest = ln.split("=")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, "no counter summary under profiles/"
+    now = decode_sources_digest()
+    if digest != now:
+        return None, "counter summary %s was taken at kernel sources %s, this run has %s: not reported" % (
+            TRAFFIC_PROFILE, digest, now)
+    return value, "%s (rocprofv3 --pmc, copy-calibrated; taken at kernel sources %s = this run's)" % (TRAFFIC_PROFILE, digest)
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -230,10 +254,14 @@ def _paged_case(torch, dev, lens, seed, shared_prefix=None, hq=16, hkv=8, d=128,
     return w, own
 
 
-def other_decode_configs(pa, torch, dev, launches):
+OTHER_CONFIGS = ("cfg1", "cfg3_p512", "cfg3_auto", "cfg4", "cfg4_shared_prefix")
+
+
+def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
     """Decode launches of the first, third and fourth benchmark configuration (FP16 KV, 16 q / 8 kv
     heads x 128, block 16; context lengths from the same seeds as the parity tests).  Median of
-    REPEATS x `launches` launches, all three alternated in one timed loop."""
+    REPEATS x `launches` launches, all alternated in one timed loop.  `which`: the launches to run
+    (a profiler run names one, so that every kernel name in its trace stands for one workload)."""
     HQ, HKV, D, BS = 16, 8, 128, 16
     scale = D ** -0.5
     row = HKV * D * 2 * 2                                   # K and V bytes of one token, fp16
@@ -295,12 +323,14 @@ def other_decode_configs(pa, torch, dev, launches):
                                       "choice) read once per prompt, matrix kernel + merge" % pg4.partition_size,
                                       kv_bytes=sum(lens4) * row, unique_kv_bytes=unique_tokens * row)
 
+    fns = {k: v for k, v in fns.items() if k in which}
+    meta = {k: v for k, v in meta.items() if k in which}
     t = time_alternating(torch, fns, launches)
     # the merge pass of the two config-3 splits alone, inside a replayed graph (device time)
     lib = pa._native.load()
     merge_us = {}
     for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3)):
-        if not psz:
+        if not psz or name not in which:
             continue
         parts = (width3 + psz - 1) // psz
         nbytes = lib.pa_workspace_bytes(4, HQ, D, parts)
@@ -502,7 +532,7 @@ def mfma_ceiling(pa, torch, dev):
     return out
 
 
-def kv_store_times(pa, torch, dev, steps, warmup):
+def kv_store_times(pa, torch, dev, steps, warmup, token_counts=(64, 4096)):
     """Paged KV-cache write of one decode step (64 new tokens) and of one prefill chunk (4096
     tokens), FP16 copy and FP8 quantising store, into random slots of a pool.  Device time per call
     inside a replayed HIP graph (16 calls per graph: eagerly a call costs its own launch, ~11 us
@@ -512,7 +542,7 @@ def kv_store_times(pa, torch, dev, steps, warmup):
     HKV, D, BS, NB = 8, 128, 16, 4096 // 16 + 64
     g = torch.Generator(device=dev).manual_seed(7)
     out = {}
-    for n in (64, 4096):
+    for n in token_counts:
         k = torch.randn(n, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
         v = torch.randn(n, HKV, D, generator=g, device=dev, dtype=torch.float32).half()
         slots = torch.randperm(NB * BS, generator=g, device=dev)[:n].to(torch.int32)
@@ -533,7 +563,7 @@ def kv_store_times(pa, torch, dev, steps, warmup):
         rec = {"fp16_us": round(g16 * 1e3, 2), "fp8_us": round(g8 * 1e3, 2),
                "fp16_eager_us": round(ms16 * 1e3, 2), "fp8_eager_us": round(ms8 * 1e3, 2),
                "fp16_algorithmic_bytes": bytes16, "fp8_algorithmic_bytes": bytes8}
-        if n == 4096:
+        if n >= 4096:
             rec["fp16_gbps"] = round(bytes16 / g16 / 1e6, 1)
             rec["fp8_gbps"] = round(bytes8 / g8 / 1e6, 1)
             rec["fp16_frac_of_8TBps"] = round(bytes16 / g16 / 1e6 / HBM_PEAK_GBPS, 4)
@@ -854,10 +884,14 @@ def main():
     ap.add_argument("--sections", default="all",
                     help="comma-separated parts to run: headline (the FP16 / FP8 launches), probe (the same "
                          "launches with loads only), others (configs 1, 3, 4), gqa (wider query groups), prefill, "
-                         "extras, cpu; 'all' = every one.  For profiler runs, which want one kind of launch "
+                         "extras, cpu, stores (the KV-cache write alone; also part of extras); 'all' = every one.  For profiler runs, which want one kind of launch "
                          "per kernel name: the load probe is the decode kernel itself with a flag set, and the "
                          "other configurations launch the headline's kernels on other shapes.  Without "
                          "`headline` the run prints a reduced line for the parts it ran")
+    ap.add_argument("--others", default=",".join(OTHER_CONFIGS),
+                    help="the launches of the others section (a profiler run names one)")
+    ap.add_argument("--store-tokens", default="64,4096",
+                    help="token counts of the stores section (the KV-cache write alone; a profiler run names one)")
     ap.add_argument("--gqa", default="4,8,4fp8,8fp8",
                     help="the launches of the gqa section: GQA ratios over 8 KV heads, 'fp8' appended for an FP8 cache "
                          "(a profiler run names one, so that the kernel name stands for one workload)")
@@ -873,12 +907,12 @@ def main():
 
     sections = set(args.sections.split(","))
     if "all" in sections:
-        sections = {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}
+        sections = {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}      # stores: part of extras
     if args.no_extras:
         sections.discard("extras")
     if args.no_cpu_baseline:
         sections.discard("cpu")
-    unknown = sections - {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}
+    unknown = sections - {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu", "stores"}
     if unknown:
         print("bench.py: unknown section(s) %s" % sorted(unknown), file=sys.stderr)
         sys.exit(2)
@@ -893,11 +927,14 @@ def main():
         if args.copy_calibration:
             copy_calibration(torch, dev)
         if "others" in sections:
-            part["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+            part["other_configs"] = other_decode_configs(pa, torch, dev, launches, args.others.split(","))
         if "gqa" in sections:
             part["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
         if "prefill" in sections:
             part["prefill_mfma"] = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup))
+        if "stores" in sections:
+            part["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup,
+                                              [int(x) for x in args.store_tokens.split(",")])
         print(json.dumps(part))
         return
     probe_only = "headline" not in sections and "cpu" not in sections
@@ -1007,6 +1044,7 @@ def main():
     prefill = prefill_cfg5a(pa, torch, dev, launches, max(20, args.warmup)) if "prefill" in sections else None
     f16, f8 = results["fp16"], results["fp8"]
     speedup = med(f16["us"]) / med(f8["us"])
+    traffic16, traffic8 = measured_traffic("traffic_bytes_fp16"), measured_traffic("traffic_bytes_fp8")
     line = {
         "metric": "paged decode attn achieved HBM GB/s (% peak) + us/step at bs=64 ctx=4k",
         "value": round(f16["gbps"], 1),
@@ -1051,11 +1089,11 @@ def main():
             "frac": round(f16["kernel_gbps"] / HBM_PEAK_GBPS, 4),
             "kernel_us": spread(f16["kernel_us"]),
             "algorithmic_bytes": f16["bytes"],
-            "traffic": measured_traffic("traffic_bytes_fp16") if (B, CTX) == (64, 4096) else None,
-            "traffic_source": "profiles/paged_decode_bs64_ctx4096_pmc_traffic.txt (rocprofv3 --pmc, copy-calibrated)",
+            "traffic": traffic16[0] if (B, CTX) == (64, 4096) else None,
+            "traffic_source": traffic16[1],
             "fp8_kernel": {"achieved": round(f8["kernel_gbps"], 1), "frac": round(f8["kernel_gbps"] / HBM_PEAK_GBPS, 4),
                            "algorithmic_bytes": f8["bytes"],
-                           "traffic": measured_traffic("traffic_bytes_fp8") if (B, CTX) == (64, 4096) else None},
+                           "traffic": traffic8[0] if (B, CTX) == (64, 4096) else None},
         },
     }
     if "probe" in sections:
@@ -1071,7 +1109,7 @@ def main():
         line["roofline"]["frac_of_plain_stream_read"] = round(f16["kernel_gbps"] / stream_read["best_gbps"], 4)
         line["roofline"]["fp8_kernel"]["frac_of_plain_stream_read"] = round(f8["kernel_gbps"] / stream_read["best_gbps"], 4)
     if "others" in sections:
-        line["other_configs"] = other_decode_configs(pa, torch, dev, launches)
+        line["other_configs"] = other_decode_configs(pa, torch, dev, launches, args.others.split(","))
     if "gqa" in sections:
         line["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
     if prefill is not None:
