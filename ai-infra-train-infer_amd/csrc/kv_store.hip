@@ -118,14 +118,18 @@ __global__ __launch_bounds__(256) void kv_store_fp8_kernel(
   const float s = __fmul_rn(__fdiv_rn(1.0f, amax), 448.0f);
   if (lane == 0) *scale_dst = s;
 
+  // The scaled values never exceed 448 by more than a rounding (the largest element times 448 / amax),
+  // and on that range - and for NaN - the hardware conversion (v_cvt_pk_fp8_f32: OCP e4m3fn on gfx950,
+  // round to nearest even, subnormals, signed zero) gives the bytes of the reference's cast; what it does
+  // beyond 464, where the reference's cast makes NaN, cannot be reached from here.
   auto encode_store = [&](const float(&x)[16], int64_t e) {
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      uint32_t b = 0;
-#pragma unroll
-      for (int k = 0; k < 4; ++k) b |= f32_to_e4m3fn(__fmul_rn(x[4 * i + k], s)) << (8 * k);
-      w[i] = b;
+      int b = 0;
+      b = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[4 * i], s), __fmul_rn(x[4 * i + 1], s), b, false);
+      b = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[4 * i + 2], s), __fmul_rn(x[4 * i + 3], s), b, true);
+      w[i] = (uint32_t)b;
     }
     *(uint4*)(dst + e) = make_uint4(w[0], w[1], w[2], w[3]);
   };

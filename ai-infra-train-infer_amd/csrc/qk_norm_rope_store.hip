@@ -102,10 +102,11 @@ __device__ __forceinline__ uint2 encode8(const float (&x)[8], float s) {
   uint32_t w[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    uint32_t b = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) b |= f32_to_e4m3fn(__fmul_rn(x[4 * j + k], s)) << (8 * k);
-    w[j] = b;
+    // the hardware conversion, as in kv_store_fp8_kernel (same bytes on the range the scale allows)
+    int b = 0;
+    b = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[4 * j], s), __fmul_rn(x[4 * j + 1], s), b, false);
+    b = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[4 * j + 2], s), __fmul_rn(x[4 * j + 3], s), b, true);
+    w[j] = (uint32_t)b;
   }
   return make_uint2(w[0], w[1]);
 }
