@@ -29,6 +29,8 @@ DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
             f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-function",
             "-I", INCLUDE, "-I", CSRC, "-I", PROBES, "-Rpass-analysis=kernel-resource-usage"] + DEVICE_FLAGS
+# extra compiler flags (e.g. -DNAME=value for a tuning macro of a kernel), space separated
+CXXFLAGS += os.environ.get("PA_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def _hipcc():
