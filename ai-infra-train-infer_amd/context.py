@@ -30,6 +30,11 @@ class InferenceContext:
     # physical blocks, as attention.prepare_prefix_groups() returns them (a PrefixGroups); None = read
     # every row alone
     prefix_groups: Optional[object] = None
+    # decode, optional (no counterpart in the reference): what the host knows about context_lens - an
+    # upper bound on the longest row and the mean - so that the attention launch is sized for the rows
+    # instead of for the width of the block table (attention.choose_partition); 0 = unknown
+    longest_context_len: int = 0
+    mean_context_len: float = 0.0
 
 
 _CONTEXT = InferenceContext()
@@ -45,6 +50,8 @@ def set_context(
     context_lens: Optional[torch.Tensor] = None,
     block_tables: Optional[torch.Tensor] = None,
     prefix_groups: Optional[object] = None,
+    longest_context_len: int = 0,
+    mean_context_len: float = 0.0,
 ):
     """Install the context for the next model forward."""
     global _CONTEXT
@@ -58,6 +65,8 @@ def set_context(
         context_lens=context_lens,
         block_tables=block_tables,
         prefix_groups=prefix_groups,
+        longest_context_len=longest_context_len,
+        mean_context_len=mean_context_len,
     )
 
 

@@ -207,6 +207,78 @@ struct Tile {
   float vs[G::RL];
 };
 
+// Partitions of a row that hold tokens.
+__device__ __forceinline__ int live_partitions(const DecodeParams& p, int row) {
+  const int ctx = p.context_lens[row];
+  return ctx <= 0 ? 0 : min((ctx + p.partition_size - 1) / p.partition_size, p.max_partitions);
+}
+
+// ... and how many of them are whole (the last one is not when the row ends inside it).
+__device__ __forceinline__ int whole_partitions(const DecodeParams& p, int row) {
+  const int ctx = p.context_lens[row];
+  return ctx <= 0 ? 0 : min(ctx / p.partition_size, p.max_partitions);
+}
+
+// Lane l holds `mine`, a count for rows l * per_lane ... l * per_lane + per_lane - 1; count(row) gives
+// one row's.  Finds the row that holds item u of the concatenation of all rows' items, and u's index
+// inside that row; false when there are `total` <= u items.
+template <typename Count>
+__device__ __forceinline__ bool locate_item(int mine, int u, int lane, int per_lane, Count count, int& row, int& index,
+                                            int& total) {
+  int upto = mine;   // items of the rows of lanes 0 ... lane
+  for (int d = 1; d < 64; d <<= 1) {
+    const int t = __shfl_up(upto, d, 64);
+    if (lane >= d) upto += t;
+  }
+  total = __shfl(upto, 63, 64);
+  const unsigned long long past = __ballot(upto > u);
+  if (past == 0) return false;
+  const int owner = __ffsll(past) - 1;
+  int base = __shfl(upto - mine, owner, 64);
+  int r = owner * per_lane;
+  // the owner's rows hold more than u - base items, so the walk ends inside them
+  for (int i = 1; i < per_lane; ++i) {
+    const int c = count(r);
+    if (u < base + c) break;
+    base += c;
+    ++r;
+  }
+  row = r;
+  index = u - base;
+  return true;
+}
+
+// Work unit u of a partitioned launch -> (row, partition).  The grid is sized for batch x
+// max_partitions units, but the units are the (row, partition) pairs that hold tokens: first the
+// whole partitions, row by row, then the rows' last, shorter ones.  A ragged batch so packs its work
+// into the first workgroups, the rest - one run at the end of the grid - leave at once (workgroups
+// without work BETWEEN working ones are what costs: they hold the slots of a dispatch round that others
+// wait for), and the short pieces come last, where they fill the gaps the long ones leave on the CUs.
+// Every wave works the mapping out for itself, from the context lengths alone: lane l counts the
+// partitions of rows l * k ... l * k + k - 1 (k = ceil(batch / 64)), a wave-wide running sum finds the
+// lane whose rows hold unit u, a walk over that lane's rows the row.  False: u lies beyond the work of
+// this launch.
+__device__ __forceinline__ bool unit_to_row_partition(const DecodeParams& p, int u, int lane, int& row, int& part) {
+  const int per_lane = (p.batch + 63) >> 6;
+  const int first = lane * per_lane;
+  int whole = 0, tails = 0;
+  for (int i = 0; i < per_lane; ++i)
+    if (first + i < p.batch) {
+      const int w = whole_partitions(p, first + i);
+      whole += w;
+      tails += live_partitions(p, first + i) - w;
+    }
+  int total_whole;
+  if (locate_item(whole, u, lane, per_lane, [&](int r) { return whole_partitions(p, r); }, row, part, total_whole))
+    return true;
+  int index, total_tails;
+  if (!locate_item(tails, u - total_whole, lane, per_lane,
+                   [&](int r) { return live_partitions(p, r) - whole_partitions(p, r); }, row, index, total_tails))
+    return false;
+  part = whole_partitions(p, row);     // the partition after the whole ones
+  return true;
+}
+
 // W waves per workgroup in QS groups of WQ = W / QS.  Lane layout inside a wave: lane = 8 g + j,
 // j the 16-byte piece of a row, g the row group; hs = g % HPW picks the KV head, tr = g / HPW
 // the token of a row load.
@@ -262,8 +334,10 @@ __global__ __launch_bounds__(W * 64) void paged_decode_kernel(const DecodeParams
     in = slot % p.inner;
     u = (slot / p.inner) * 8 + (x & 7);
   }
-  const int part = u % p.max_partitions;
-  const int b = u / p.max_partitions;
+  int part = 0, b = u;
+  if (p.max_partitions > 1 && !unit_to_row_partition(p, u, lane, b, part)) return;
+  b = __builtin_amdgcn_readfirstlane(b);
+  part = __builtin_amdgcn_readfirstlane(part);
   const int gq = p.num_q_heads / p.num_kv_heads;
   const int kv_groups = p.num_kv_heads / HPW;
   const int kvg = in % kv_groups;

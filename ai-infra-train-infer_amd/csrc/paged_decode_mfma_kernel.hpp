@@ -199,8 +199,13 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
   } else {
     in = blockIdx.x % p.inner;
     const int u = blockIdx.x / p.inner;
-    part = u % p.max_partitions;
-    b = u / p.max_partitions;
+    part = 0;
+    b = u;
+    if (p.max_partitions > 1) {
+      if (!unit_to_row_partition(p, u, threadIdx.x & 63, b, part)) return;
+      b = __builtin_amdgcn_readfirstlane(b);
+      part = __builtin_amdgcn_readfirstlane(part);
+    }
   }
   const int kvg = in % kv_groups;
   const int sub = in / kv_groups;

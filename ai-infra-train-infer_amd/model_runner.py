@@ -56,6 +56,15 @@ class ModelRunnerConfig:
     # keeps the last step's groups for as long as the batch's first blocks stay what they were.
     share_prefix_decode: bool = True
     prefix_partition_sizes: Tuple[int, ...] = (1024, 512)     # tokens; coarsest first
+    # Recorded decode launches cannot be resized, and one sized for the width of the block tables
+    # (max_num_blocks) is a poor fit for a batch of rows a fraction of that long.  Graphs over a
+    # DecodeState are therefore recorded per context bucket - launches sized for rows of up to that many
+    # tokens - and a step replays the smallest bucket that holds its longest row (the host knows the
+    # lengths).  None: the table's width and every quarter of the one before down to 2048 tokens.
+    decode_context_buckets: Optional[Tuple[int, ...]] = None
+    # also record, where the launch policy would shape it differently, a graph for ragged batches (rows
+    # half as long as the bucket on average), replayed when the mean length is below 0.7 of the bucket
+    ragged_decode_graphs: bool = True
 
 
 def slots_for_range(block_table, start, end, block_size):
@@ -128,6 +137,15 @@ class DecodeState:
 
     def active_rows(self) -> List[int]:
         return np.flatnonzero(self._lens).tolist()
+
+    def known_lengths(self, batch: Optional[int] = None) -> Tuple[int, float]:
+        """(longest, mean) context length over the first `batch` rows (default: the rows in use), free
+        rows counted as 0: what the host knows without asking the device."""
+        n = self.rows_in_use if batch is None else int(batch)
+        if n <= 0:
+            return 0, 0.0
+        lens = self._lens[:n]
+        return int(lens.max()), float(lens.sum()) / n
 
     def num_tokens(self, row: int) -> int:
         return int(self._lens[row])
@@ -238,17 +256,22 @@ class DecodeState:
                 cursor += 1
         self._groups_dev.copy_(host.pin_memory(), non_blocking=True)
 
-    def prefix_groups(self, batch: int, partition_size: Optional[int] = None, for_graph: bool = False):
+    def prefix_groups(self, batch: int, partition_size: Optional[int] = None, for_graph: bool = False,
+                      longest_context: Optional[int] = None):
         """PrefixGroups over the state's device descriptors for the first `batch` rows, or None when
         no rows share a prefix.  for_graph: the descriptors at their full capacity whatever they hold
         now (empty groups cost a workgroup that returns at once), for partition_size - what a
-        recorded launch must be sized with."""
+        recorded launch must be sized with; longest_context: the rows the launch will serve hold at
+        most that many tokens (a prefix cannot be longer than the rows that share it)."""
         from .attention import PrefixGroups
         if not self.tracks_prefixes:
             return None
         if for_graph:
             size = int(partition_size)
-            parts = -(-self.max_blocks * self.block_size // size)
+            tokens = self.max_blocks * self.block_size
+            if longest_context:
+                tokens = min(tokens, int(longest_context))
+            parts = -(-tokens // size)
             return PrefixGroups(size, self._group_desc, self._group_rows, self._row_skip[:batch], self.max_groups,
                                 self.max_group_rows, parts, 0)
         self.sync_prefix_groups()
@@ -325,19 +348,29 @@ class DecodeState:
         self._fresh_rows.clear()
 
     def set_context(self, batch: Optional[int] = None, share_prefixes: bool = True,
-                    graph_partition_size: Optional[int] = None):
+                    graph_partition_size: Optional[int] = None, lengths="host"):
         """Point the attention layers at the first `batch` rows (default: the rows in use).
         share_prefixes: hand them the groups of rows that share a prefix, when there are any;
         graph_partition_size: the descriptors at full capacity for that partition size instead (what
-        a graph is recorded over)."""
+        a graph is recorded over).  lengths: what the launches may assume about the rows - "host": the
+        lengths the host has counted (an eager step), (longest, mean): these (a recorded launch serves
+        every batch that fits them; mean 0 = rows as long as the longest), None: nothing beyond the
+        width of the tables."""
         n = self.rows_in_use if batch is None else batch
+        if isinstance(lengths, str):
+            longest, mean = self.known_lengths(n)
+        elif lengths is None:
+            longest, mean = 0, 0.0
+        else:
+            longest, mean = int(lengths[0]), float(lengths[1])
         groups = None
         if graph_partition_size is not None:
-            groups = self.prefix_groups(n, graph_partition_size, for_graph=True)
+            groups = self.prefix_groups(n, graph_partition_size, for_graph=True, longest_context=longest or None)
         elif share_prefixes:
             groups = self.prefix_groups(n)
         set_context(False, slot_mapping=self.slot_mapping[:n], context_lens=self.context_lens[:n],
-                    block_tables=self.block_tables[:n], prefix_groups=groups)
+                    block_tables=self.block_tables[:n], prefix_groups=groups,
+                    longest_context_len=longest, mean_context_len=mean)
         return n
 
 
@@ -357,13 +390,15 @@ class ModelRunner:
         self._graph_pool = None
         self._graph_vars: Optional[Dict[str, torch.Tensor]] = None
         self._graph_batch_sizes: List[int] = []
-        self._state_graphs: Dict[Tuple[int, int, Optional[int]], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        # (id of the DecodeState, batch size, shared-prefix partition size or None, context bucket, for ragged batches)
+        self._state_graphs: Dict[tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._state_buckets: Dict[int, List[int]] = {}      # id of the DecodeState -> context buckets recorded, ascending
         self._hf_model: Optional[torch.nn.Module] = None
-        self._state_graph_lookup: Dict[Tuple[int, int, Optional[int]], object] = {}
+        self._state_graph_lookup: Dict[tuple, object] = {}
         self._prefix_groups_kept = None          # (signature of the batch, PrefixGroups or None) of the last decode step
         # how run_decode_state ran its steps: replays of a graph recorded over the shared-prefix launch,
         # replays of a plain graph, eager forwards
-        self.decode_state_stats = {"shared_prefix_graph": 0, "plain_graph": 0, "eager": 0}
+        self.decode_state_stats = {"shared_prefix_graph": 0, "plain_graph": 0, "ragged_graph": 0, "eager": 0}
 
     # ---------------------------------------------------------------- cache binding
 
@@ -543,6 +578,9 @@ class ModelRunner:
             context_lens=self._to_device(lens, torch.int32),
             block_tables=self._prepare_block_tables(sequences),
             prefix_groups=groups,
+            # the host has the lengths: the attention launch is sized for these rows, not for full tables
+            longest_context_len=int(lens.max()) if n else 0,
+            mean_context_len=float(lens.mean()) if n else 0.0,
         )
         return self._to_device(ids, torch.long), self._to_device(pos, torch.long)
 
@@ -813,13 +851,43 @@ class ModelRunner:
     # ---------------------------------------------------------------- decode over a DecodeState
 
     @torch.inference_mode()
-    def capture_decode_state_graphs(self, state: DecodeState, batch_sizes: Optional[List[int]] = None):
+    def _context_buckets(self, state: DecodeState) -> List[int]:
+        """Context buckets (tokens, ascending) that graphs over `state` are recorded for; the last one is
+        the width of its block tables."""
+        width = state.max_blocks * state.block_size
+        given = getattr(self.config, "decode_context_buckets", None)
+        if given is None:
+            buckets, b = [], width
+            while b >= 2048:
+                buckets.append(b)
+                b //= 4
+        else:
+            buckets = [int(b) for b in given if 0 < int(b) < width]
+        return sorted(set(buckets) | {width})
+
+    def _ragged_launch_differs(self, bs: int, bucket: int) -> bool:
+        """Whether the launch policy shapes a ragged batch of `bs` rows of up to `bucket` tokens
+        differently from a full one (only then is a second graph worth recording)."""
+        from .attention import choose_partition
+        cfg = self.config
+        elem = 1 if self._cache_dtype == "fp8" else 2
+        full = choose_partition(bs, cfg.num_heads, cfg.num_kv_heads, bucket, cfg.head_dim, elem)
+        ragged = choose_partition(bs, cfg.num_heads, cfg.num_kv_heads, bucket, cfg.head_dim, elem,
+                                  mean_context=0.5 * bucket)
+        return full != ragged
+
+    def capture_decode_state_graphs(self, state: DecodeState, batch_sizes: Optional[List[int]] = None,
+                                    context_buckets: Optional[List[int]] = None):
         """Record the decode forward over the first n rows of `state` for each n: the graph's
-        inputs are the state's own tensors, so a replay needs no copies at all.  When the state keeps
-        groups of rows that share a prefix (and config.share_prefix_decode), a second graph per n and
-        partition size is recorded over its group descriptors - at their full capacity, empty groups
-        included, since a recorded launch cannot be resized - and run_decode_state replays that one
-        whenever the state holds a group."""
+        inputs are the state's own tensors, so a replay needs no copies at all.
+
+        A recorded launch cannot be resized, so each n is recorded per context bucket (launches sized for
+        rows of up to that many tokens; default: config.decode_context_buckets) and, where the launch
+        policy would split a ragged batch differently from a full one, once more for ragged batches;
+        run_decode_state replays the graph that fits the lengths the host has counted.  When the state
+        keeps groups of rows that share a prefix (and config.share_prefix_decode), one more graph per n,
+        bucket and partition size is recorded over its group descriptors - at their full capacity, empty
+        groups included - and replayed whenever the state holds a group."""
         from .attention import sizing_graph_workspace
         if not torch.cuda.is_available() or self.model is None:
             return
@@ -827,35 +895,56 @@ class ModelRunner:
             batch_sizes = sorted({b for b in (1, 2, 4, 8, 16, 32, 64, 128, 256) if b < state.max_batch}
                                  | {state.max_batch})
         self._reserve_decode_workspace(max(batch_sizes))
-        variants = [None]
+        width = state.max_blocks * state.block_size
+        if context_buckets is None:
+            buckets = self._context_buckets(state)
+        else:
+            buckets = sorted({int(b) for b in context_buckets if 0 < int(b) < width} | {width})
+        self._state_buckets[id(state)] = sorted(set(self._state_buckets.get(id(state), [])) | set(buckets))
+        prefix_sizes = []
         if state.tracks_prefixes and getattr(self.config, "share_prefix_decode", False):
-            variants += list(state.prefix_partition_sizes)
+            prefix_sizes = list(state.prefix_partition_sizes)
         for bs in sorted(batch_sizes, reverse=True):
-            for psize in variants:
-                if psize is not None and bs < 2:
-                    continue
-                state.set_context(bs, share_prefixes=False, graph_partition_size=psize)
-                with sizing_graph_workspace():
-                    self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, pool=self._graph_pool):
-                    out = self.model(state.input_ids[:bs], positions=state.positions[:bs])
-                if self._graph_pool is None:
-                    self._graph_pool = graph.pool()
-                self._state_graphs[(id(state), bs, psize)] = (graph, out)
-                self._state_graph_lookup.clear()
-                torch.cuda.synchronize()
-                reset_context()
+            for bucket in buckets:
+                variants = [(None, False)]
+                if getattr(self.config, "ragged_decode_graphs", True) and self._ragged_launch_differs(bs, bucket):
+                    variants.append((None, True))
+                if bs >= 2:
+                    variants += [(psize, False) for psize in prefix_sizes if psize <= bucket]
+                for psize, ragged in variants:
+                    lengths = (bucket, 0.5 * bucket if ragged else 0.0)
+                    state.set_context(bs, share_prefixes=False, graph_partition_size=psize, lengths=lengths)
+                    with sizing_graph_workspace():
+                        self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, pool=self._graph_pool):
+                        out = self.model(state.input_ids[:bs], positions=state.positions[:bs])
+                    if self._graph_pool is None:
+                        self._graph_pool = graph.pool()
+                    self._state_graphs[(id(state), bs, psize, bucket, ragged)] = (graph, out)
+                    self._state_graph_lookup.clear()
+                    torch.cuda.synchronize()
+                    reset_context()
 
-    def _state_graph_for(self, state, rows, partition_size):
-        """The graph recorded over `state` for the smallest batch size >= rows (and the given shared-prefix
-        partition size, None = the plain launch), or None."""
-        key = (id(state), rows, partition_size)
+    def _state_graph_for(self, state, rows, partition_size, longest=0, mean=0.0):
+        """The graph recorded over `state` for the smallest batch size >= rows and the smallest context
+        bucket >= longest (for the given shared-prefix partition size, None = the plain launch; the one
+        for ragged batches when there is one and `mean` is below 0.7 of the bucket), or None."""
+        bucket = next((b for b in self._state_buckets.get(id(state), ()) if b >= longest), None)
+        if bucket is None:
+            return None
+        ragged = partition_size is None and 0 < mean < 0.7 * bucket
+        key = (id(state), rows, partition_size, bucket, ragged)
         hit = self._state_graph_lookup.get(key, False)
         if hit is False:
-            sizes = sorted(bs for (sid, bs, ps) in self._state_graphs if sid == id(state) and ps == partition_size and bs >= rows)
-            hit = self._state_graphs[(id(state), sizes[0], partition_size)] if sizes else None
+            hit = None
+            for flavour in ((True, False) if ragged else (False,)):
+                sizes = sorted(bs for (sid, bs, ps, bk, rg) in self._state_graphs
+                               if sid == id(state) and ps == partition_size and bk == bucket and rg == flavour and bs >= rows)
+                if sizes:
+                    hit = self._state_graphs[(id(state), sizes[0], partition_size, bucket, flavour)] + (flavour,)
+                    break
             self._state_graph_lookup[key] = hit
         return hit
 
@@ -867,14 +956,16 @@ class ModelRunner:
         n = state.rows_in_use
         share = getattr(self.config, "share_prefix_decode", False)
         state.sync_prefix_groups()
-        if self.config.enable_cuda_graph:
+        if self.config.enable_cuda_graph and id(state) in self._state_buckets:
             psize = state.prefix_partition_size if share else None
+            longest, mean = state.known_lengths(n)
             for want in ((psize, None) if psize is not None else (None,)):
-                hit = self._state_graph_for(state, n, want)
+                hit = self._state_graph_for(state, n, want, longest, mean)
                 if hit is not None:
-                    graph, out = hit
+                    graph, out, ragged = hit
                     graph.replay()
-                    self.decode_state_stats["plain_graph" if want is None else "shared_prefix_graph"] += 1
+                    self.decode_state_stats["shared_prefix_graph" if want is not None else
+                                            "ragged_graph" if ragged else "plain_graph"] += 1
                     return out[:n]
         self.decode_state_stats["eager"] += 1
         state.set_context(n, share_prefixes=share)
@@ -886,6 +977,7 @@ class ModelRunner:
         """Drop every recorded graph (after a weight update)."""
         self._state_graphs.clear()
         self._state_graph_lookup.clear()
+        self._state_buckets.clear()
         self._prefix_groups_kept = None
         self._graphs.clear()
         self._graph_outputs.clear()

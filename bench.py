@@ -254,7 +254,7 @@ def _paged_case(torch, dev, lens, seed, shared_prefix=None, hq=16, hkv=8, d=128,
     return w, own
 
 
-OTHER_CONFIGS = ("cfg1", "cfg3_p512", "cfg3_auto", "cfg4", "cfg4_shared_prefix")
+OTHER_CONFIGS = ("cfg1", "cfg3_p512", "cfg3_auto", "cfg3_known_lengths", "cfg4", "cfg4_shared_prefix")
 
 
 def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
@@ -294,8 +294,13 @@ def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
                                                w3["context_lens"], scale, partition_size=512, out=w3["out"])
     fns["cfg3_auto"] = lambda: pa.paged_decode(w3["q"], w3["k_cache"], w3["v_cache"], w3["block_tables"],
                                                w3["context_lens"], scale, out=w3["out"])
+    # ... and at the split the policy picks when the caller passes the lengths the host has
+    known3 = dict(longest_context=max(lens3), mean_context=sum(lens3) / 4.0)
+    p3k, _ = pa.choose_partition(4, HQ, HKV, width3, D, 2, pa.attention._compute_units(dev), **known3)
+    fns["cfg3_known_lengths"] = lambda: pa.paged_decode(w3["q"], w3["k_cache"], w3["v_cache"], w3["block_tables"],
+                                                        w3["context_lens"], scale, out=w3["out"], **known3)
     kv3 = sum(lens3) * row
-    for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3)):
+    for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3), ("cfg3_known_lengths", p3k)):
         nparts = sum((n + psz - 1) // psz for n in lens3) if psz else 0
         meta[name] = dict(workload="batch 4, ctx U[16384,32768] (seed 1003), FP16 KV, partition size %d" % psz,
                           kv_bytes=kv3, partials_bytes=2 * HQ * nparts * (D + 2) * 4,
@@ -329,7 +334,7 @@ def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
     # the merge pass of the two config-3 splits alone, inside a replayed graph (device time)
     lib = pa._native.load()
     merge_us = {}
-    for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3)):
+    for name, psz in (("cfg3_p512", 512), ("cfg3_auto", p3), ("cfg3_known_lengths", p3k)):
         if not psz or name not in which:
             continue
         parts = (width3 + psz - 1) // psz
@@ -363,6 +368,49 @@ def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
             rec.update(kv_bytes=m["kv_bytes"], partials_bytes_written_and_read=m["partials_bytes"],
                        partitions_launched=m["partitions_launched"], gbps=round(total / us / 1e3, 1),
                        frac_of_8TBps=round(total / us / 1e3 / HBM_PEAK_GBPS, 4))
+        out[name] = rec
+    return out
+
+
+def ragged_decode_configs(pa, torch, dev, launches):
+    """Batches of rows of unequal length under block tables wider than the rows (a serving batch: the
+    table is as wide as the longest request allowed, the rows are wherever their requests are).
+    FP16 KV, 16 q / 8 kv heads x 128, block 16.  Each batch is launched with the shape the policy picks
+    from the table's width alone and with the shape it picks when the caller passes what it knows about
+    the rows (longest_context / mean_context: the model runner has the lengths on the host); the rate
+    counts the tokens the rows hold."""
+    HQ, HKV, D, BS = 16, 8, 128, 16
+    scale = D ** -0.5
+    row = HKV * D * 2 * 2
+    fns, meta, keep = {}, {}, []
+    for name, batch, lo, hi, width_tokens in (("b64_ctx256_4096", 64, 256, 4096, 4096), ("b64_ctx256_4096_tables32k", 64, 256, 4096, 32768),
+                                              ("b16_ctx1024_8192_tables32k", 16, 1024, 8192, 32768),
+                                              ("b256_ctx64_1024_tables32k", 256, 64, 1024, 32768)):
+        lens = _uniform_lens(torch, 5, batch, lo, hi)
+        w, _ = _paged_case(torch, dev, lens, 7)
+        tables = torch.zeros(batch, max(width_tokens // BS, w["block_tables"].shape[1]), dtype=torch.int32, device=dev)
+        tables[:, :w["block_tables"].shape[1]] = w["block_tables"]
+        keep.append((w, tables))
+        longest, mean = max(lens), sum(lens) / batch
+        width = tables.shape[1] * BS
+        cus = pa.attention._compute_units(dev)
+        fns[name + "/table_width"] = lambda w=w, tables=tables: pa.paged_decode(
+            w["q"], w["k_cache"], w["v_cache"], tables, w["context_lens"], scale, out=w["out"])
+        fns[name + "/known_lengths"] = lambda w=w, tables=tables, longest=longest, mean=mean: pa.paged_decode(
+            w["q"], w["k_cache"], w["v_cache"], tables, w["context_lens"], scale, out=w["out"],
+            longest_context=longest, mean_context=mean)
+        meta[name] = dict(workload="batch %d, ctx U[%d,%d] (seed 5), tables %d tokens wide" % (batch, lo, hi, width),
+                          kv_bytes=sum(lens) * row,
+                          split_from_table_width=list(pa.choose_partition(batch, HQ, HKV, width, D, 2, cus)),
+                          split_from_known_lengths=list(pa.choose_partition(batch, HQ, HKV, width, D, 2, cus, longest, mean)))
+    t = time_alternating(torch, fns, launches)
+    out = {}
+    for name, m in meta.items():
+        rec = dict(m)
+        for how in ("table_width", "known_lengths"):
+            us = med(t[name + "/" + how])
+            rec[how] = {"us": spread(t[name + "/" + how]), "gbps": round(m["kv_bytes"] / us / 1e3, 1),
+                        "frac_of_8TBps": round(m["kv_bytes"] / us / 1e3 / HBM_PEAK_GBPS, 4)}
         out[name] = rec
     return out
 
@@ -883,7 +931,7 @@ def main():
                     help="launches per timed repeat are max(steps, this); profiler runs with counters lower it")
     ap.add_argument("--sections", default="all",
                     help="comma-separated parts to run: headline (the FP16 / FP8 launches), probe (the same "
-                         "launches with loads only), others (configs 1, 3, 4), gqa (wider query groups), prefill, "
+                         "launches with loads only), others (configs 1, 3, 4), ragged (rows of unequal length under wide tables), gqa (wider query groups), prefill, "
                          "extras, cpu, stores (the KV-cache write alone; also part of extras); 'all' = every one.  For profiler runs, which want one kind of launch "
                          "per kernel name: the load probe is the decode kernel itself with a flag set, and the "
                          "other configurations launch the headline's kernels on other shapes.  Without "
@@ -907,12 +955,12 @@ def main():
 
     sections = set(args.sections.split(","))
     if "all" in sections:
-        sections = {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu"}      # stores: part of extras
+        sections = {"headline", "probe", "others", "ragged", "gqa", "prefill", "extras", "cpu"}      # stores: part of extras
     if args.no_extras:
         sections.discard("extras")
     if args.no_cpu_baseline:
         sections.discard("cpu")
-    unknown = sections - {"headline", "probe", "others", "gqa", "prefill", "extras", "cpu", "stores"}
+    unknown = sections - {"headline", "probe", "others", "ragged", "gqa", "prefill", "extras", "cpu", "stores"}
     if unknown:
         print("bench.py: unknown section(s) %s" % sorted(unknown), file=sys.stderr)
         sys.exit(2)
@@ -928,6 +976,8 @@ def main():
             copy_calibration(torch, dev)
         if "others" in sections:
             part["other_configs"] = other_decode_configs(pa, torch, dev, launches, args.others.split(","))
+        if "ragged" in sections:
+            part["ragged_decode"] = ragged_decode_configs(pa, torch, dev, launches)
         if "gqa" in sections:
             part["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
         if "prefill" in sections:
@@ -1110,6 +1160,8 @@ def main():
         line["roofline"]["fp8_kernel"]["frac_of_plain_stream_read"] = round(f8["kernel_gbps"] / stream_read["best_gbps"], 4)
     if "others" in sections:
         line["other_configs"] = other_decode_configs(pa, torch, dev, launches, args.others.split(","))
+    if "ragged" in sections:
+        line["ragged_decode"] = ragged_decode_configs(pa, torch, dev, launches)
     if "gqa" in sections:
         line["gqa_decode"] = gqa_decode_configs(pa, torch, dev, launches, args.gqa.split(","))
     if prefill is not None:

@@ -293,6 +293,55 @@ def test_launch_policy_splits_and_head_pairing_keep_the_result(pa, lib, gpu, cac
         check(gpu_decode(pa, c, gpu, kv_heads_per_wave=hpw, waves=8), want, cache)
 
 
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+@pytest.mark.parametrize("hq", [16, 32])
+@pytest.mark.parametrize("batch", [3, 64, 65, 150, 300])
+def test_ragged_batches_pack_their_partitions(pa, gpu, cache, hq, batch):
+    """A partitioned launch numbers only the (row, partition) pairs that hold tokens and every
+    workgroup finds its pair from the context lengths: rows of very different lengths, empty rows
+    between them, more rows than a wave has lanes (each lane then counts several rows), extra table
+    columns (workgroups beyond the work), on the vector and the matrix kernel."""
+    gen = torch.Generator().manual_seed(batch * 7 + hq)
+    lens = torch.randint(1, 700, (batch,), generator=gen)
+    lens[torch.rand(batch, generator=gen) < 0.2] = 0               # empty rows anywhere
+    lens[int(torch.randint(0, batch, (1,), generator=gen))] = 1500  # one long row
+    lens = lens.tolist()
+    c = cases.make_case(batch + hq, lens, sum((n + 15) // 16 for n in lens) + 5, num_heads=hq, cache=cache, extra_cols=9)
+    want = oracle_decode(c)
+    for psize in (128, 256, 368):
+        got = gpu_decode(pa, c, gpu, partition_size=psize)
+        live = torch.tensor(lens) > 0
+        check(got[live], want[live], cache)
+        assert not got[~live].any(), "an empty row is a zero row"
+
+
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+def test_known_lengths_size_the_launch_and_never_change_the_result(pa, gpu, cache):
+    """longest_context / mean_context only shape the launch: right, too small (rows longer than the
+    bound end in the last partition) or absurd, the output is the oracle's."""
+    lens = [900, 40, 2500, 1300, 7, 1999]
+    c = cases.make_case(77, lens, sum((n + 15) // 16 for n in lens) + 5, cache=cache, extra_cols=300)   # tables 7300 tokens wide
+    want = oracle_decode(c)
+    for longest, mean in ((2500, 1124.0), (2500, None), (1000, 500.0), (256, 10.0), (10 ** 6, 10.0 ** 6), (None, 1124.0)):
+        check(gpu_decode(pa, c, gpu, longest_context=longest, mean_context=mean), want, cache)
+        check(gpu_decode(pa, c, gpu, partition_size=512, longest_context=longest), want, cache)
+    width = c["block_tables"].shape[1] * 16
+    elem = 1 if cache == "fp8" else 2
+    blind = pa.choose_partition(len(lens), 16, 8, width, 128, elem)
+    told = pa.choose_partition(len(lens), 16, 8, width, 128, elem, longest_context=2500, mean_context=1124.0)
+    assert told[0] * told[1] < blind[0] * blind[1], "the launch is sized for the rows, not for the table"
+    # the layers take the same hints from the context
+    d = cases.to_device(c, gpu)
+    for cls in (pa.PagedAttention, pa.PartitionedPagedAttention):
+        attn = cls(16, 8, 128, cache_dtype=cache)
+        attn.k_cache, attn.v_cache, attn.k_scale, attn.v_scale = d["k_cache"], d["v_cache"], d["k_scale"], d["v_scale"]
+        pa.set_context(False, context_lens=d["context_lens"], block_tables=d["block_tables"],
+                       longest_context_len=2500, mean_context_len=1124.0)
+        got = attn._decode_attention(d["q"], pa.get_context()).cpu()
+        pa.reset_context()
+        check(got, want, cache)
+
+
 def test_table_check_counts_what_the_kernels_would_clamp(pa, gpu, monkeypatch):
     c = cases.make_case(60, [100, 40, 0, 33], 32)
     d = cases.to_device(c, gpu)

@@ -166,6 +166,71 @@ def test_decode_loop_over_the_state_equals_the_prepare_decode_path(pa, gpu, grap
     pa.reset_context()
 
 
+def test_graphs_per_context_bucket_follow_the_rows(pa, gpu):
+    """Tables far wider than the rows: graphs are recorded per context bucket (and, where the launch
+    policy splits ragged batches differently, per flavour), each step replays the smallest bucket that
+    holds the longest row, and the logits are those of the prepare_decode path whichever graph ran."""
+    from test_gpu_model import Session, small_model
+    model = small_model(pa, seed=19)
+    ref = Session(pa, model, gpu, num_blocks=160)
+    dev = Session(pa, model, gpu, num_blocks=160, graphs=None)
+    dev.runner.config.enable_cuda_graph = True
+    g = torch.Generator().manual_seed(20)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist() for n in (9, 700, 17, 300)]
+    for p in prompts:
+        ref.add(p)
+        dev.add(p)
+    first = ref.prefill()[0].argmax(-1).tolist()
+    assert dev.prefill()[0].argmax(-1).tolist() == first
+    st = pa.DecodeState(8, 128, 16, dev.pool.num_blocks, device=gpu)            # tables of 2048 tokens
+    rows = [st.admit(s["block_table"], len(s["token_ids"]), t) for s, t in zip(dev.seqs, first)]
+    # at the benchmark shape a ragged batch of 64 rows is split where a full one is read in one pass (256
+    # rows are read in one pass either way); the test asks for the second graph of one bucket itself
+    big = pa.ModelRunner(None, pa.ModelRunnerConfig(num_heads=16, num_kv_heads=8, head_dim=128))
+    assert big._ragged_launch_differs(64, 4096) and not big._ragged_launch_differs(256, 1024)
+    dev.runner._ragged_launch_differs = lambda bs, bucket: bucket == 710
+    dev.runner.capture_decode_state_graphs(st, [4, 8], context_buckets=[256, 710, 1024])
+    assert dev.runner._state_buckets[id(st)] == [256, 710, 1024, 2048]
+    recorded = {(bs, bk, rg) for (_, bs, ps, bk, rg) in dev.runner._state_graphs}
+    assert {(4, 256, False), (4, 710, False), (4, 1024, False), (4, 2048, False), (8, 2048, False)} <= recorded
+    assert {(4, 710, True), (8, 710, True)} == {x for x in recorded if x[2]}
+    assert torch.equal(dev.pool.kv_cache_tensor, ref.pool.kv_cache_tensor)     # capture wrote nothing
+    seen = []
+    real_for = dev.runner._state_graph_for
+
+    def spy(state, n, want, longest=0, mean=0.0):
+        hit = real_for(state, n, want, longest, mean)
+        bucket = next(b for b in dev.runner._state_buckets[id(state)] if b >= longest)
+        seen.append((bucket, hit[2]))
+        return hit
+    dev.runner._state_graph_for = spy
+    toks, next_dev, live = first, None, list(rows)
+    for step in range(24):
+        if step == 16:                      # the long row leaves: the batch fits a smaller bucket again
+            st.retire(1)
+            live.remove(1)
+        want = ref.decode(toks)
+        grants = {}
+        for r in st.rows_needing_block():
+            dev.seqs[r]["block_table"].append(dev.free.pop())
+            grants[r] = dev.seqs[r]["block_table"][-1]
+        st.step(grants or None, next_dev)
+        assert st.known_lengths()[0] == max(len(ref.seqs[r]["token_ids"]) for r in live)
+        got = dev.runner.run_decode_state(st)
+        torch.testing.assert_close(got[live].float().cpu(), want[live].float().cpu(), rtol=2e-3, atol=2e-3)
+        next_dev = pa.sample_tokens(got, temperature=0.0)
+        toks = want.argmax(-1).tolist()
+        assert [next_dev.tolist()[r] for r in live] == [toks[r] for r in live]
+        _ = (want.float() @ want.float().t()).sum().item()              # eager work between replays
+    buckets = [b for b, _ in seen]
+    assert buckets[0] == 710 and 1024 in buckets and buckets[-1] == 710 and 2048 not in buckets and 256 not in buckets
+    assert buckets.index(1024) == 710 - 701 + 1                          # the step whose longest row reaches 711 tokens
+    stats = dev.runner.decode_state_stats
+    assert stats["eager"] == 0 and stats["plain_graph"] + stats["ragged_graph"] == 24
+    assert stats["ragged_graph"] == sum(1 for _, rg in seen if rg) > 0   # rows of 10 ... 700 tokens: ragged
+    pa.reset_context()
+
+
 def test_state_keeps_prefix_groups_through_admits_and_retires(pa, gpu):
     """Host side of the group bookkeeping: rebuilt when a row is admitted or retired, never by a step; the
     device descriptors hold what the host list says."""

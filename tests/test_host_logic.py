@@ -66,6 +66,37 @@ def test_choose_partition_policy(pa):
     assert not f(100, True) and not f(512, False) and f(4096, True)
 
 
+def test_choose_partition_with_known_lengths(pa):
+    """What the host knows about the rows sizes the launch: a bound on the longest row replaces the
+    table's width, a mean well below it says the batch is ragged (finer split: partitions without
+    tokens cost nothing, partitions with tokens spread evenly)."""
+    cp = pa.choose_partition
+    kl = pa.attention._known_lengths
+    assert kl(4096, None, None) == (4096, None)
+    assert kl(32768, 4000, None) == (4096, None)          # rounded up to 256 tokens
+    assert kl(4096, 10 ** 6, None) == (4096, None)        # never beyond the table
+    assert kl(4096, 4096, 2048.0) == (4096, 8) and kl(4096, 4096, 3000.0) == (4096, None)
+    assert kl(4096, 4096, 1.0) == (4096, 1)
+    # a wide table with short rows is the narrow table
+    assert cp(64, 16, 8, 32768, longest_context=4096) == cp(64, 16, 8, 4096)
+    assert cp(16, 16, 8, 32768, longest_context=8000) == cp(16, 16, 8, 8192)
+    # full rows at the headline shape: one pass; ragged ones: split into a few hundred tokens
+    assert cp(64, 16, 8, 4096, mean_context=4000.0) == (0, 1)
+    p, n = cp(64, 16, 8, 4096, mean_context=2176.0)
+    assert n == -(-4096 // p) and 384 <= p <= 1024 and p % 128 == 0
+    p_full, n_full = cp(16, 16, 8, 16384)
+    p_rag, n_rag = cp(16, 16, 8, 16384, mean_context=9200.0)
+    assert n_rag > n_full and 384 <= p_rag < p_full
+    # enough rows even out by themselves
+    assert cp(256, 16, 8, 1024, mean_context=540.0) == (0, 1)
+    # never finer than 384 tokens, never more than 128 partitions
+    assert cp(2, 16, 8, 4096, mean_context=2000.0)[0] == 384
+    p, n = cp(1, 16, 8, 131072, mean_context=50000.0)
+    assert n <= 128 and p * n >= 131072
+    # hints that say nothing change nothing
+    assert cp(36, 16, 8, 8192, longest_context=0, mean_context=0) == cp(36, 16, 8, 8192)
+
+
 def test_block_pool_layout(pa):
     pool = pa.BlockPool(4, 16, 2, 8, 128, dtype=torch.float16, device="cpu", cache_dtype="fp8")
     assert tuple(pool.kv_cache_tensor.shape) == (2, 2, 4, 16, 8, 128)
