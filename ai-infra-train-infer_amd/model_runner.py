@@ -60,11 +60,16 @@ class ModelRunnerConfig:
     # (max_num_blocks) is a poor fit for a batch of rows a fraction of that long.  Graphs over a
     # DecodeState are therefore recorded per context bucket - launches sized for rows of up to that many
     # tokens - and a step replays the smallest bucket that holds its longest row (the host knows the
-    # lengths).  None: the table's width and every quarter of the one before down to 2048 tokens.
+    # lengths).  None: the table's width and every half of the one before down to 2048 tokens.
     decode_context_buckets: Optional[Tuple[int, ...]] = None
     # also record, where the launch policy would shape it differently, a graph for ragged batches (rows
-    # half as long as the bucket on average), replayed when the mean length is below 0.7 of the bucket
+    # 0.45 of the bucket long on average), replayed when the mean length is below 0.7 of the bucket
     ragged_decode_graphs: bool = True
+
+
+# mean row length, as a share of the context bucket, that the graphs for ragged batches are recorded for
+# (rows between a quarter of the bucket and the whole of it: batches with longer rows take the next bucket)
+_RAGGED_GRAPH_MEAN = 0.45
 
 
 def slots_for_range(block_table, start, end, block_size):
@@ -860,7 +865,7 @@ class ModelRunner:
             buckets, b = [], width
             while b >= 2048:
                 buckets.append(b)
-                b //= 4
+                b //= 2
         else:
             buckets = [int(b) for b in given if 0 < int(b) < width]
         return sorted(set(buckets) | {width})
@@ -873,7 +878,7 @@ class ModelRunner:
         elem = 1 if self._cache_dtype == "fp8" else 2
         full = choose_partition(bs, cfg.num_heads, cfg.num_kv_heads, bucket, cfg.head_dim, elem)
         ragged = choose_partition(bs, cfg.num_heads, cfg.num_kv_heads, bucket, cfg.head_dim, elem,
-                                  mean_context=0.5 * bucket)
+                                  mean_context=_RAGGED_GRAPH_MEAN * bucket)
         return full != ragged
 
     def capture_decode_state_graphs(self, state: DecodeState, batch_sizes: Optional[List[int]] = None,
@@ -912,7 +917,7 @@ class ModelRunner:
                 if bs >= 2:
                     variants += [(psize, False) for psize in prefix_sizes if psize <= bucket]
                 for psize, ragged in variants:
-                    lengths = (bucket, 0.5 * bucket if ragged else 0.0)
+                    lengths = (bucket, _RAGGED_GRAPH_MEAN * bucket if ragged else 0.0)
                     state.set_context(bs, share_prefixes=False, graph_partition_size=psize, lengths=lengths)
                     with sizing_graph_workspace():
                         self.model(state.input_ids[:bs], positions=state.positions[:bs])     # library handles, allocator warm-up

@@ -825,6 +825,69 @@ def model_step_cfg5b(pa, torch, dev, steps, warmup):
     return out
 
 
+def model_step_ragged(pa, torch, dev, steps=12):
+    """A serving batch through the caller: 64 sequences of U[256, 4000] tokens in a DecodeState whose block
+    tables are 32768 tokens wide (the longest request allowed), a Qwen3-0.6B-shaped model (28 layers,
+    random weights), FP16 KV.  One step = advance kernel + replayed graph + greedy sampling on the device.
+    First with graphs recorded for the tables' width and full rows only, then with the runner's default:
+    one graph per context bucket, and per bucket one for ragged batches where the launch differs; each
+    step replays the graph that fits the lengths the state has counted on the host."""
+    import time as _time
+    cfg = pa.Qwen3PagedConfig()
+    BS, B, WIDTH = 16, 64, 32768 // 16
+    lens = [min(x, 4000) for x in _uniform_lens(torch, 5, B, 256, 4096)]     # the timed steps stay inside the 4096-token bucket
+    spare = 2
+    nb = sum((x + BS - 1) // BS + spare for x in lens) + 64
+    torch.manual_seed(11)
+    with torch.device(dev):
+        model = pa.Qwen3PagedModel(cfg).half().eval()
+    pool = pa.BlockPool(nb, BS, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim, dtype=torch.float16, device=dev)
+    pool.kv_cache_tensor.normal_()
+    runner = pa.ModelRunner(model, pa.ModelRunnerConfig(
+        num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads, head_dim=cfg.head_dim,
+        hidden_size=cfg.hidden_size, block_size=BS, max_num_blocks=WIDTH, device="cuda:0", enable_cuda_graph=True,
+        max_cuda_graph_batch_size=B))
+    runner.bind_kv_cache(pool.kv_cache_tensor)
+    state = pa.DecodeState(B, WIDTH, BS, nb, device=dev)
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(6)).tolist()
+    at = 0
+    for n in lens:
+        need = (n + BS - 1) // BS + spare
+        state.admit(perm[at:at + need], n, 1)
+        at += need
+    out = {"workload": "Qwen3-0.6B shape, 28 layers, batch 64, ctx U[256,4096] capped at 4000 (seed 5), block tables 32768 tokens wide, "
+                       "FP16 KV, one decode step"}
+    nxt = [None]
+    for label, buckets, ragged in (("graphs_for_table_width", [], False), ("graphs_per_context_bucket", None, True)):
+        runner.invalidate_cuda_graphs()
+        runner.config.ragged_decode_graphs = ragged
+        runner.capture_decode_state_graphs(state, [B], context_buckets=buckets)
+        before = dict(runner.decode_state_stats)
+        for _ in range(2):
+            state.step(None, nxt[0])
+            nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
+        torch.cuda.synchronize()
+        t0 = _time.perf_counter()
+        host = 0.0
+        for _ in range(steps):
+            h0 = _time.perf_counter()
+            state.step(None, nxt[0])
+            logits = runner.run_decode_state(state)
+            host += _time.perf_counter() - h0
+            nxt[0] = pa.sample_tokens(logits, temperature=0.0)
+        torch.cuda.synchronize()
+        taken = {k: v - before[k] for k, v in runner.decode_state_stats.items() if v != before[k]}
+        assert taken.get("eager", 0) == 0, taken
+        out[label] = {"step_ms": round((_time.perf_counter() - t0) * 1e3 / steps, 3),
+                      "host_us_per_step": round(host * 1e6 / steps, 1),
+                      "buckets_recorded": runner._state_buckets[id(state)], "graphs_replayed": taken}
+    out["known_lengths"] = list(state.known_lengths())
+    runner.invalidate_cuda_graphs()
+    del pool, model, state
+    torch.cuda.empty_cache()
+    return out
+
+
 def model_step_cfg4(pa, torch, dev, steps=12):
     """Fourth benchmark configuration through the caller: 32 prompts x 8 samples in one DecodeState of 256
     rows, the samples aliasing their prompt's 64 blocks through the cache manager
@@ -1184,6 +1247,7 @@ def main():
         line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
         line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
         line["model_decode_step_cfg4"] = model_step_cfg4(pa, torch, dev)
+        line["model_decode_step_ragged"] = model_step_ragged(pa, torch, dev)
     if "cpu" in results:
         line["cpu_baseline"] = results["cpu"]
     print(json.dumps(line))
