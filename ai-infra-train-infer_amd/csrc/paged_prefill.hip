@@ -294,6 +294,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
 
   const int bs_mask = (1 << p.bs_log2) - 1;
   const int64_t token_elems = p.block_tables ? (int64_t)p.num_kv_heads * D : p.kv_token_stride;
+  const uint32_t row_bytes = (uint32_t)(token_elems * ES);      // bytes between consecutive tokens (the host checks the range)
   const int32_t* bt_row = p.block_tables ? p.block_tables + seq * p.bt_stride : nullptr;
   const int bt_last = max((int)p.bt_stride - 1, 0);
 
@@ -365,7 +366,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
           const int key0 = t * kBN + (NT * c) / CPR + wave * (64 / CPR);   // first row of this wave's instruction
           const int phys = min(max(__builtin_amdgcn_readlane(ids, c), 0), p.num_blocks - 1);
           const int64_t slot0 = ((int64_t)phys << p.bs_log2) + (key0 & bs_mask);
-          const int64_t base = slot0 * token_elems * ES;
+          const uint64_t base = (uint64_t)(uint32_t)slot0 * row_bytes;     // both below 2^32: one 32 x 32 -> 64 multiply
           move_chunk(c, buf, uniform_ptr(p.k + base) + lane_part[c], uniform_ptr(p.v + base) + lane_part[c], slot0 + lane / CPR);
         }
       } else {
@@ -373,7 +374,7 @@ __global__ __launch_bounds__(64 * W, (W == 4 ? 2 : 1)) void paged_prefill_kernel
         for (int c = 0; c < NCH; ++c) {
           const int key0 = t * kBN + (NT * c) / CPR + wave * (64 / CPR);
           const int64_t slot0 = (int64_t)k0 + key0;
-          const int64_t base = slot0 * token_elems * ES;
+          const uint64_t base = (uint64_t)(uint32_t)slot0 * row_bytes;
           move_chunk(c, buf, uniform_ptr(p.k + base) + lane_part[c], uniform_ptr(p.v + base) + lane_part[c], slot0 + lane / CPR);
         }
       }
@@ -716,6 +717,10 @@ extern "C" int pa_prefill(const void* q, int q_dtype, int64_t q_token_stride, co
   }
   if (num_seqs > 65535 || max_seqlen_q > 65535 * 64)
     return fail(PA_ERR_UNSUPPORTED, "pa_prefill: too many sequences or query tokens for one launch");
+  // the kernel multiplies a token's slot by the bytes between tokens as two 32-bit numbers
+  if (num_blocks * block_size >= (int64_t(1) << 32) || kv_token_stride >= (int64_t(1) << 30) ||
+      num_kv_heads * head_dim >= (int64_t(1) << 30))
+    return fail(PA_ERR_UNSUPPORTED, "pa_prefill: pool of 2^32 slots or more, or 2^30 elements or more between tokens");
 
   const int g = (int)(num_q_heads / num_kv_heads);
   const int hpwg = (g % 2 == 0) ? 2 : 1;
