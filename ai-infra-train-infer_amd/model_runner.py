@@ -390,8 +390,9 @@ class ModelRunner:
         self._kv_cache: Optional[torch.Tensor] = None
         self._k_scale = self._v_scale = None
         self._cache_dtype = "fp16"
-        self._graphs: Dict[int, torch.cuda.CUDAGraph] = {}
-        self._graph_outputs: Dict[int, torch.Tensor] = {}
+        self._graphs: Dict[tuple, torch.cuda.CUDAGraph] = {}      # (batch size, context bucket, for ragged batches)
+        self._graph_outputs: Dict[tuple, torch.Tensor] = {}
+        self._graph_buckets: List[int] = []
         self._graph_pool = None
         self._graph_vars: Optional[Dict[str, torch.Tensor]] = None
         self._graph_batch_sizes: List[int] = []
@@ -786,8 +787,15 @@ class ModelRunner:
     # ---------------------------------------------------------------- decode graphs
 
     @torch.inference_mode()
-    def capture_cuda_graphs(self, batch_sizes: Optional[List[int]] = None):
-        """Record one HIP graph of the decode forward per batch size over shared static inputs."""
+    def capture_cuda_graphs(self, batch_sizes: Optional[List[int]] = None,
+                            context_buckets: Optional[List[int]] = None):
+        """Record HIP graphs of the decode forward over shared static inputs: one per batch size
+        (src/inference/model_runner.py:710-760) and, because the static block tables are max_num_blocks
+        wide whatever the batch holds, per context bucket (launches sized for rows of up to that many
+        tokens; default config.decode_context_buckets) and, where the launch policy cuts a ragged batch
+        differently, once more for ragged batches.  A step replays the graph that fits the lengths
+        prepare_decode has passed on (InferenceContext.longest_context_len / mean_context_len); a context
+        without them takes the graph sized for the tables' width."""
         if not torch.cuda.is_available() or self.model is None:
             return
         if batch_sizes is None:
@@ -798,6 +806,8 @@ class ModelRunner:
         max_bs = max(batch_sizes)
         dev = self.config.device
         self._reserve_decode_workspace(max_bs)
+        width = self.config.max_num_blocks * self.block_size
+        self._graph_buckets = self._buckets_for_width(width, context_buckets)
         gv = {
             "input_ids": torch.zeros(max_bs, dtype=torch.long, device=dev),
             "positions": torch.zeros(max_bs, dtype=torch.long, device=dev),
@@ -806,21 +816,30 @@ class ModelRunner:
             "block_tables": torch.zeros(max_bs, self.config.max_num_blocks, dtype=torch.int32, device=dev),
         }
         for bs in reversed(self._graph_batch_sizes):
-            graph = torch.cuda.CUDAGraph()
-            set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
-                        block_tables=gv["block_tables"][:bs])
-            # warm-up outside the capture: library handles, allocator warm-up
-            with sizing_graph_workspace():
-                self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
-            torch.cuda.synchronize()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                out = self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
-            self._graphs[bs] = graph
-            self._graph_outputs[bs] = out
-            torch.cuda.synchronize()
-            reset_context()
+            for bucket in self._graph_buckets:
+                flavours = [False]
+                if getattr(self.config, "ragged_decode_graphs", True) and self._ragged_launch_differs(bs, bucket):
+                    flavours.append(True)
+                for ragged in flavours:
+                    graph = torch.cuda.CUDAGraph()
+                    hints = dict(longest_context_len=bucket if bucket < width else 0,
+                                 mean_context_len=_RAGGED_GRAPH_MEAN * bucket if ragged else 0.0)
+                    set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
+                                block_tables=gv["block_tables"][:bs], **hints)
+                    # warm-up outside the capture: library handles, allocator warm-up
+                    with sizing_graph_workspace():
+                        self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
+                    torch.cuda.synchronize()
+                    set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
+                                block_tables=gv["block_tables"][:bs], **hints)
+                    with torch.cuda.graph(graph, pool=self._graph_pool):
+                        out = self.model(gv["input_ids"][:bs], positions=gv["positions"][:bs])
+                    if self._graph_pool is None:
+                        self._graph_pool = graph.pool()
+                    self._graphs[(bs, bucket, ragged)] = graph
+                    self._graph_outputs[(bs, bucket, ragged)] = out
+                    torch.cuda.synchronize()
+                    reset_context()
         self._graph_vars = gv
 
     def _reserve_decode_workspace(self, max_batch):
@@ -834,10 +853,16 @@ class ModelRunner:
 
     def _run_with_cuda_graph(self, input_ids, positions):
         bs = input_ids.size(0)
-        graph_bs = next((x for x in self._graph_batch_sizes if x >= bs), None)
-        if graph_bs is None or graph_bs not in self._graphs:
-            return self.model(input_ids, positions=positions)
         ctx = get_context()
+        graph_bs = next((x for x in self._graph_batch_sizes if x >= bs), None)
+        # the smallest context bucket that holds the longest row the host knows of (none known: the widest)
+        longest = getattr(ctx, "longest_context_len", 0) or self._graph_buckets[-1]
+        bucket = next((b for b in self._graph_buckets if b >= longest), None)
+        mean = getattr(ctx, "mean_context_len", 0.0)
+        ragged = bucket is not None and 0 < mean < 0.7 * bucket and (graph_bs, bucket, True) in self._graphs
+        key = (graph_bs, bucket, ragged)
+        if graph_bs is None or key not in self._graphs:
+            return self.model(input_ids, positions=positions)
         gv = self._graph_vars
         gv["input_ids"][:bs] = input_ids
         gv["positions"][:bs] = positions
@@ -850,17 +875,18 @@ class ModelRunner:
         if ctx.block_tables is not None:
             bt = ctx.block_tables
             gv["block_tables"][:bs, :bt.size(1)] = bt    # the tail stays stale, as in the reference
-        self._graphs[graph_bs].replay()
-        return self._graph_outputs[graph_bs][:bs]
+        self._graphs[key].replay()
+        return self._graph_outputs[key][:bs]
 
     # ---------------------------------------------------------------- decode over a DecodeState
 
     @torch.inference_mode()
-    def _context_buckets(self, state: DecodeState) -> List[int]:
-        """Context buckets (tokens, ascending) that graphs over `state` are recorded for; the last one is
-        the width of its block tables."""
-        width = state.max_blocks * state.block_size
-        given = getattr(self.config, "decode_context_buckets", None)
+    def _buckets_for_width(self, width: int, given=None) -> List[int]:
+        """Context buckets (tokens, ascending) for block tables `width` tokens wide; the last one is the
+        width.  given None: config.decode_context_buckets, and without those the width and every half
+        of the one before down to 2048 tokens."""
+        if given is None:
+            given = getattr(self.config, "decode_context_buckets", None)
         if given is None:
             buckets, b = [], width
             while b >= 2048:
@@ -869,6 +895,10 @@ class ModelRunner:
         else:
             buckets = [int(b) for b in given if 0 < int(b) < width]
         return sorted(set(buckets) | {width})
+
+    def _context_buckets(self, state: DecodeState) -> List[int]:
+        """Context buckets that graphs over `state` are recorded for."""
+        return self._buckets_for_width(state.max_blocks * state.block_size)
 
     def _ragged_launch_differs(self, bs: int, bucket: int) -> bool:
         """Whether the launch policy shapes a ragged batch of `bs` rows of up to `bucket` tokens
@@ -901,10 +931,7 @@ class ModelRunner:
                                  | {state.max_batch})
         self._reserve_decode_workspace(max(batch_sizes))
         width = state.max_blocks * state.block_size
-        if context_buckets is None:
-            buckets = self._context_buckets(state)
-        else:
-            buckets = sorted({int(b) for b in context_buckets if 0 < int(b) < width} | {width})
+        buckets = self._buckets_for_width(width, context_buckets)
         self._state_buckets[id(state)] = sorted(set(self._state_buckets.get(id(state), [])) | set(buckets))
         prefix_sizes = []
         if state.tracks_prefixes and getattr(self.config, "share_prefix_decode", False):

@@ -52,7 +52,7 @@ def small_model(pa, cache_dtype="fp16", partition_size=0, seed=0, fused_qk=True)
 class Session:
     """Minimal host bookkeeping for the test: a block table per sequence from a free list."""
 
-    def __init__(self, pa, model, gpu, num_blocks=64, cache_dtype="fp16", graphs=None):
+    def __init__(self, pa, model, gpu, num_blocks=64, cache_dtype="fp16", graphs=None, max_num_blocks=16, buckets=None):
         cfg = model.cfg
         self.pa, self.bs = pa, 16
         self.gpu_model = copy.deepcopy(model).half().to(gpu)
@@ -61,11 +61,11 @@ class Session:
         self.runner = pa.ModelRunner(self.gpu_model, pa.ModelRunnerConfig(
             num_layers=cfg.num_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
             head_dim=cfg.head_dim, hidden_size=cfg.hidden_size, vocab_size=cfg.vocab_size, block_size=16,
-            max_num_blocks=16, device="cuda:0", enable_cuda_graph=graphs is not None))
+            max_num_blocks=max_num_blocks, device="cuda:0", enable_cuda_graph=graphs is not None))
         self.runner.bind_kv_cache(self.pool.kv_cache_tensor, self.pool.k_scale, self.pool.v_scale,
                                   self.pool.cache_dtype)
         if graphs:
-            self.runner.capture_cuda_graphs(graphs)
+            self.runner.capture_cuda_graphs(graphs, context_buckets=buckets)
         self.free = list(range(num_blocks))[::-1]
         self.seqs = []
 
@@ -187,6 +187,46 @@ def test_graph_replay_equals_eager_on_every_replay(pa, gpu):
                            eager.pool.kv_cache_tensor[:, :, eager.seqs[1]["block_table"][0]].cpu())
         # eager work between replays
         _ = (le.float() @ le.float().t()).sum().item()
+
+
+def test_graphs_per_context_bucket_under_wide_static_tables(pa, gpu):
+    """The static block tables of the recorded graphs are max_num_blocks wide; prepare_decode passes the
+    lengths it has, and the step replays the graph recorded for the smallest context bucket that holds
+    them (and the one for ragged batches where there is one) - with the logits of the eager path."""
+    model = small_model(pa, seed=8)
+    eager = Session(pa, model, gpu, num_blocks=120, max_num_blocks=128)
+    graph = Session(pa, model, gpu, num_blocks=120, max_num_blocks=128, graphs=None)
+    graph.runner.config.enable_cuda_graph = True
+    graph.runner._ragged_launch_differs = lambda bs, bucket: bucket == 512
+    graph.runner.capture_cuda_graphs([4], context_buckets=[256, 512])
+    assert graph.runner._graph_buckets == [256, 512, 2048]
+    assert sorted(graph.runner._graphs) == [(4, 256, False), (4, 512, False), (4, 512, True), (4, 2048, False)]
+    g = torch.Generator().manual_seed(9)
+    prompts = [torch.randint(0, 512, (n,), generator=g).tolist() for n in (9, 250, 17)]
+    for p in prompts:
+        eager.add(p)
+        graph.add(p)
+    close(graph.prefill()[0], eager.prefill()[0].cpu(), 1e-3)
+    replayed = []
+    for key, gr in graph.runner._graphs.items():
+        real = gr.replay
+        gr.replay = (lambda key=key, real=real: (replayed.append(key), real())[1])
+    for step in range(10):                   # the longest row passes 256 tokens on the way: 251 ... 260
+        nxt = torch.randint(0, 512, (3,), generator=g).tolist()
+        le = eager.decode(nxt)
+        lg = graph.decode(nxt)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(lg.float().cpu(), le.float().cpu(), rtol=2e-3, atol=2e-3)
+        _ = (le.float() @ le.float().t()).sum().item()
+    # rows of 10 ... 260 tokens: mean far below 0.7 of the bucket; the 256-token bucket has no graph for ragged batches
+    assert replayed == [(4, 256, False)] * 6 + [(4, 512, True)] * 4, replayed
+    # a context without lengths (run_batch_decode: metadata already on the device) takes the widest graph
+    d = graph.seqs
+    tables = graph.runner._prepare_block_tables(d)
+    lens = torch.tensor([len(x["token_ids"]) for x in d], dtype=torch.int32, device=gpu)
+    ids = torch.tensor([x["token_ids"][-1] for x in d], device=gpu)
+    out = graph.runner.run_batch_decode(ids, (lens - 1).long(), tables, lens)
+    assert replayed[-1] == (4, 2048, False) and out.shape[0] == 3
 
 
 def test_config5b_qwen3_0p6b_shaped_decode_step(pa, gpu):
