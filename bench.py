@@ -1245,7 +1245,7 @@ def main():
         line["fused_qk_norm_rope_store"] = fused_qk_times(pa, torch, dev, args.steps, args.warmup)
         line["block_elementwise"] = block_elementwise_times(pa, torch, dev, args.steps, args.warmup)
         line["sampler"] = sampler_times(pa, torch, dev, args.steps, args.warmup)
-        line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 3))
+        line["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 10))
         line["model_decode_step_cfg4"] = model_step_cfg4(pa, torch, dev)
         line["model_decode_step_ragged"] = model_step_ragged(pa, torch, dev)
     if "cpu" in results:
