@@ -836,7 +836,7 @@ def model_step_ragged(pa, torch, dev, steps=12):
     cfg = pa.Qwen3PagedConfig()
     BS, B, WIDTH = 16, 64, 32768 // 16
     lens = [min(x, 4000) for x in _uniform_lens(torch, 5, B, 256, 4096)]     # the timed steps stay inside the 4096-token bucket
-    spare = 2
+    spare = 4
     nb = sum((x + BS - 1) // BS + spare for x in lens) + 64
     torch.manual_seed(11)
     with torch.device(dev):
@@ -863,7 +863,7 @@ def model_step_ragged(pa, torch, dev, steps=12):
         runner.config.ragged_decode_graphs = ragged
         runner.capture_decode_state_graphs(state, [B], context_buckets=buckets)
         before = dict(runner.decode_state_stats)
-        for _ in range(2):
+        for _ in range(8):
             state.step(None, nxt[0])
             nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
         torch.cuda.synchronize()
@@ -901,7 +901,7 @@ def model_step_cfg4(pa, torch, dev, steps=12):
     BS, PROMPTS, SAMPLES, PREFIX = 16, 32, 8, 1024
     suf = _uniform_lens(torch, 1004, PROMPTS * SAMPLES, 64, 512)
     lens = [PREFIX + x for x in suf]
-    spare = 2                                                # blocks per row for the tokens of the timed steps
+    spare = 4                                                # blocks per row for the tokens of the timed steps
     nb = PROMPTS * (PREFIX // BS) + sum((x + BS - 1) // BS + 1 + spare for x in suf) + 64
     torch.manual_seed(11)
     with torch.device(dev):
@@ -937,7 +937,7 @@ def model_step_cfg4(pa, torch, dev, steps=12):
     for label, share in (("shared_prefix_graph", True), ("plain_graph", False)):
         runner.config.share_prefix_decode = share
         before = dict(runner.decode_state_stats)
-        for _ in range(2):
+        for _ in range(8):
             state.step(None, nxt[0])
             nxt[0] = pa.sample_tokens(runner.run_decode_state(state), temperature=0.0)
         torch.cuda.synchronize()
@@ -958,7 +958,7 @@ def model_step_cfg4(pa, torch, dev, steps=12):
         out[label + "_host_us_per_step"] = {"DecodeState.step": round(host_step * 1e6 / steps, 1),
                                             "run_decode_state (graph launch call)": round(host_run * 1e6 / steps, 1)}
         taken = {k: runner.decode_state_stats[k] - before[k] for k in before}
-        assert taken[label] == steps + 2 and sum(taken.values()) == steps + 2, taken
+        assert taken[label] == steps + 8 and sum(taken.values()) == steps + 8, taken
     out["attention_us_saved_per_step"] = round((out["plain_graph_step_ms"] - out["shared_prefix_graph_step_ms"]) * 1e3, 1)
     runner.invalidate_cuda_graphs()
     del pool, model, state
