@@ -277,7 +277,7 @@ inline int plan_decode(const char* who, const void* q, int q_dtype, int64_t q_to
     p.ws_out = w.out;
   }
   p.inner = (int)(num_kv_heads / s.hpw) * slices;
-  p.xcd_rows = (kv == KV_FP8 && !matrix && p.inner > 1 && (batch * max_partitions) % 8 == 0) ? 1 : 0;
+  p.xcd_rows = (kv == KV_FP8 && !shared && p.inner > 1 && (batch * max_partitions) % 8 == 0) ? 1 : 0;
   p.batch = (int)batch;
   p.group_desc = nullptr;
   p.group_rows = nullptr;

@@ -198,7 +198,15 @@ __global__ __launch_bounds__(W * 64) void paged_decode_mfma_kernel(const DecodeP
     }
   } else {
     in = blockIdx.x % p.inner;
-    const int u = blockIdx.x / p.inner;
+    int u = blockIdx.x / p.inner;
+    if (p.xcd_rows) {
+      // fp8 caches: the workgroups of one (row, partition) on one XCD, where they share the row's scale
+      // lines (the same mapping as in paged_decode_kernel)
+      const int x = blockIdx.x;
+      const int slot = x >> 3;
+      in = slot % p.inner;
+      u = (slot / p.inner) * 8 + (x & 7);
+    }
     part = 0;
     b = u;
     if (p.max_partitions > 1) {
