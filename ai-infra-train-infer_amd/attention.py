@@ -530,6 +530,7 @@ def _debug_tables():
 # caches, streaming loads): the pick is within 1.5 % of the best measured split on average, 7 % at worst.
 _MIN_AUTO_PARTITION = 256          # tokens
 _MIN_RAGGED_PARTITION = 384        # tokens
+_MIN_RAGGED_BYTES = 96 << 20       # K and V bytes of a launch from which the split for ragged batches is used
 _MAX_AUTO_PARTITIONS = 128
 _HBM_BYTES_PER_NS = 6800.0
 _CU_BYTES_PER_NS = {2: 28.0, 1: 25.0}      # by cache element size
@@ -595,8 +596,10 @@ def _choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, k
     narrow = head_dim * kv_elem_bytes <= 128
     token_bytes = 2.0 * head_dim * kv_elem_bytes         # K and V of one head
     cu_rate = _CU_BYTES_PER_NS.get(kv_elem_bytes, 31.0)
-    if mean_sixteenths is not None:
-        # A ragged batch.  Partitions without tokens cost nothing (their workgroups are numbered last and
+    if mean_sixteenths is not None and \
+            batch * num_kv_heads * (max_context * mean_sixteenths / 16.0) * token_bytes >= _MIN_RAGGED_BYTES:
+        # A ragged batch (one large enough for the memory system to set the pace: below about 100 MB the
+        # fixed costs of a launch do, and the split for full rows of the bound is the better one).  Partitions without tokens cost nothing (their workgroups are numbered last and
         # leave at once) and workgroups of unequal length do not march in rounds - a CU takes the next
         # one when it is done - so what counts is that there are enough of them to even out: about four
         # per CU.  Rows that provide that by themselves are read in one pass; otherwise the partition is

@@ -90,9 +90,12 @@ def test_choose_partition_with_known_lengths(pa):
     # enough rows even out by themselves
     assert cp(256, 16, 8, 1024, mean_context=540.0) == (0, 1)
     # never finer than 384 tokens, never more than 128 partitions
-    assert cp(2, 16, 8, 4096, mean_context=2000.0)[0] == 384
+    assert cp(4, 16, 8, 16384, mean_context=7720.0)[0] == 384
     p, n = cp(1, 16, 8, 131072, mean_context=50000.0)
     assert n <= 128 and p * n >= 131072
+    # small launches (under about 100 MB of K and V) keep the split for full rows: fixed costs set their pace
+    assert cp(32, 16, 8, 1024, mean_context=626.0) == cp(32, 16, 8, 1024)
+    assert cp(2, 16, 8, 4096, mean_context=2000.0) == cp(2, 16, 8, 4096)
     # hints that say nothing change nothing
     assert cp(36, 16, 8, 8192, longest_context=0, mean_context=0) == cp(36, 16, 8, 8192)
 
