@@ -440,7 +440,8 @@ _sizing_for_graphs = 0
 @contextlib.contextmanager
 def sizing_graph_workspace():
     """While active, every partitioned decode launch also sizes the workspace that recorded graphs
-    use: wrap the warm-up runs that precede a capture in it."""
+    use, and launches are shaped as they will be inside the capture (the policy splits small launches
+    differently for eager calls): wrap the warm-up runs that precede a capture in it."""
     global _sizing_for_graphs
     _sizing_for_graphs += 1
     try:
@@ -528,7 +529,8 @@ def _debug_tables():
 # round of workgroups and 3 us + 0.03 us per partition for the merge pass, is smallest.  The rates
 # are fitted to a sweep of every split on an MI355X (batch 1..128, contexts 2k..32k, fp16 and fp8
 # caches, streaming loads): the pick is within 1.5 % of the best measured split on average, 7 % at worst.
-_MIN_AUTO_PARTITION = 256          # tokens
+_MIN_AUTO_PARTITION = 64           # tokens: the finest split (launches of a few rows: about one round of workgroups, however short)
+_SINGLE_PASS_UP_TO = {2: 256, 1: 512}   # contexts (tokens) that are never split, by cache element size
 _MIN_RAGGED_PARTITION = 384        # tokens
 _MIN_RAGGED_BYTES = 96 << 20       # K and V bytes of a launch from which the split for ragged batches is used
 _MAX_AUTO_PARTITIONS = 128
@@ -536,9 +538,17 @@ _HBM_BYTES_PER_NS = 6800.0
 _CU_BYTES_PER_NS = {2: 28.0, 1: 25.0}      # by cache element size
 _ROUND_NS = 2000.0
 _MERGE_NS = (3000.0, 30.0)         # fixed, per partition (the pass itself and the partials it re-reads)
+# An eager call (no graph) cannot return faster than the host can issue it: about 11.5 us for the call with
+# one launch, 5 us more with the merge pass behind it.  Below that, what the split saves on the device is lost.
+_EAGER_CALL_NS = (11500.0, 5000.0)
+_EAGER_CHECK_TOKENS = 32768        # batch x context up to which an eager call looks at that
+_LAUNCH_SHAPES = {}                # paged_decode's shapes -> what the policy said for them (replayed, eager)
 _DEFAULT_COMPUTE_UNITS = 256
 MATRIX_PATH_FROM_RATIO = 3         # GQA ratio from which pa_decode multiplies on the matrix cores (up to 16 query heads per workgroup)
 _CU_COUNT = {}
+
+
+_is_capturing = getattr(torch._C, "_cuda_isCurrentStreamCapturing", None) or torch.cuda.is_current_stream_capturing
 
 
 def _compute_units(device):
@@ -581,8 +591,8 @@ def _known_lengths(max_context, longest, mean):
 
 @functools.lru_cache(maxsize=4096)
 def _choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, kv_elem_bytes, compute_units,
-                      mean_sixteenths):
-    if max_context <= _MIN_AUTO_PARTITION or batch <= 0:
+                      mean_sixteenths, eager=False):
+    if max_context <= _SINGLE_PASS_UP_TO.get(kv_elem_bytes, 256) or batch <= 0:
         return 0, 1
     g = num_q_heads // num_kv_heads
     if g >= MATRIX_PATH_FROM_RATIO:
@@ -638,10 +648,16 @@ def _choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, k
         # lone rows of 128 bytes or less stream about 10% below the rest
         hbm = hbm_ns * (1.12 if narrow and heads == 1 else 1.0)
         rounds = -(-(wgs // heads) // compute_units)
-        busiest_ns = rounds * min(psize, max_context) * heads * token_bytes / cu_rate
+        # a CU pulls more when most of the others have nothing to do: 8 workgroups stream at twice the
+        # rate per CU that 256 do (measured at batch 1 to 32, contexts of 384 to 1024 tokens); from half
+        # the CUs on the fitted rate stands
+        lone = 1.0 + 0.8 * max(0.0, 1.0 - 2.0 * (wgs // heads) / float(compute_units))
+        busiest_ns = rounds * min(psize, max_context) * heads * token_bytes / (cu_rate * lone)
         cost = max(hbm, busiest_ns) + rounds * _ROUND_NS
         if parts > 1:
             cost += _MERGE_NS[0] + _MERGE_NS[1] * parts
+        if eager:
+            cost = max(cost, _EAGER_CALL_NS[0] + (_EAGER_CALL_NS[1] if parts > 1 else 0.0))
         if best is None or cost < best[0] * 0.99:        # ties go to the coarser split
             best = (cost, psize, parts)
     _, psize, parts = best
@@ -649,9 +665,9 @@ def _choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, k
 
 
 def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2,
-                     compute_units=_DEFAULT_COMPUTE_UNITS, longest_context=None, mean_context=None):
+                     compute_units=_DEFAULT_COMPUTE_UNITS, longest_context=None, mean_context=None, eager=False):
     """Partition size for a decode launch that has no caller-given one: the split of
-    `max_context` (a multiple of 16 tokens, at least 256) with the smallest modelled time.
+    `max_context` (a multiple of 16 tokens, at least 64) with the smallest modelled time.
     Returns (partition_size, max_partitions); (0, 1) means a single pass.
 
     max_context is what the block table can hold.  A caller that knows its rows (the model runner has
@@ -659,19 +675,21 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
     instead of the table's width (a row beyond it is still computed exactly, its last partition runs
     to the row's end), and mean_context tells a ragged batch from a full one - a ragged one is split
     finer, because partitions without tokens cost nothing and the partitions with tokens spread evenly
-    over the CUs where whole rows of unequal length do not."""
+    over the CUs where whole rows of unequal length do not.  eager: the launch is issued call by call,
+    not replayed from a graph, so a split also costs the host a second launch (it is then only taken
+    where the single pass would last longer than the two calls take to issue)."""
     bound, eighths = _known_lengths(max_context, longest_context, mean_context)
     return _choose_partition(batch, num_q_heads, num_kv_heads, bound, head_dim, kv_elem_bytes, compute_units,
-                             eighths)
+                             eighths, bool(eager))
 
 
 def choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2,
-                  compute_units=_DEFAULT_COMPUTE_UNITS, longest_context=None, mean_context=None):
+                  compute_units=_DEFAULT_COMPUTE_UNITS, longest_context=None, mean_context=None, eager=False):
     """(partition_size, max_partitions, kv_heads_per_wave) of a decode launch that has no
     caller-given shape; kv_heads_per_wave 0 leaves the choice between one and two KV heads per
     wave to the launch itself (the rule of pairs_kv_heads)."""
     psize, parts = choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim, kv_elem_bytes,
-                                    compute_units, longest_context, mean_context)
+                                    compute_units, longest_context, mean_context, eager)
     return psize, parts, 0
 
 
@@ -1023,9 +1041,27 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, k_scale
     max_context = tables.shape[1] * block_size
     hpw = kv_heads_per_wave
     if partition_size is None:
-        psize, parts, auto_hpw = choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim,
-                                               k_cache.element_size(), _compute_units(q.device),
-                                               longest_context, mean_context)
+        # what the policy says for this shape, replayed from a graph and (small launches that the
+        # graph would split only) issued call by call; remembered per shape: the policy's own cache
+        # still costs the host 1 us a call, which shows in the launches that last 10 us
+        key = (batch, num_q_heads, num_kv_heads, max_context, head_dim, k_cache.element_size(), q.device.index,
+               longest_context, mean_context)
+        shapes = _LAUNCH_SHAPES.get(key)
+        if shapes is None:
+            args = (batch, num_q_heads, num_kv_heads, max_context, head_dim, k_cache.element_size(),
+                    _compute_units(q.device), longest_context, mean_context)
+            replayed = choose_launch(*args)
+            small = replayed[1] > 1 and batch * max_context <= _EAGER_CHECK_TOKENS
+            shapes = (replayed, choose_launch(*args, eager=True) if small else None)
+            if len(_LAUNCH_SHAPES) >= 4096:
+                _LAUNCH_SHAPES.clear()
+            _LAUNCH_SHAPES[key] = shapes
+        psize, parts, auto_hpw = shapes[0]
+        # outside a graph capture the second launch of a split costs the host more than the split saves
+        # on the device (a warm-up inside sizing_graph_workspace() stands for the capture that follows:
+        # the same split)
+        if shapes[1] is not None and not _sizing_for_graphs and not _is_capturing():
+            psize, parts, auto_hpw = shapes[1]
         if hpw is None:
             hpw = auto_hpw
     else:
@@ -1211,10 +1247,10 @@ class PartitionedPagedAttention(PagedAttention):
     sized from the block-table width instead, so no host synchronisation happens: sequences
     shorter than one partition simply own a single partition, which merges to itself.
 
-    partition_size is the finest split the layer will use.  The merge is exact, so when the
-    batch already fills the GPU with coarser partitions (or with none) the launch takes those:
-    at 256 sequences a split into 512-token partitions only adds partial results to write and
-    merge.  `adaptive = False` keeps every launch at exactly partition_size.
+    The merge is exact, so the split is the launch policy's to choose (choose_partition): none at
+    256 sequences, where 512-token partitions only add partial results to write and merge; 64 to
+    128 tokens for one or two sequences, where a round of short workgroups beats a few long ones.
+    `adaptive = False` keeps every launch at exactly partition_size, the reference's split.
     """
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -1235,16 +1271,9 @@ class PartitionedPagedAttention(PagedAttention):
         shared = self._shared_prefix_decode(q, ctx, ks, vs)
         if shared is not None:
             return shared
-        psize = self.partition_size
         longest = getattr(ctx, "longest_context_len", 0) or None
         mean = getattr(ctx, "mean_context_len", 0) or None
-        if self.adaptive:
-            max_context = ctx.block_tables.shape[1] * self.k_cache.shape[1]
-            auto, _ = choose_partition(q.shape[0], self.num_heads, self.num_kv_heads, max_context,
-                                       self.head_dim, self.k_cache.element_size(), _compute_units(q.device),
-                                       longest, mean)
-            if auto == 0 or auto >= psize:
-                psize = None          # the launch's own choice: single pass or coarser partitions
+        psize = None if self.adaptive else self.partition_size      # None: the launch policy's split
         return paged_decode(q, self.k_cache, self.v_cache, ctx.block_tables, ctx.context_lens,
                             self.scale, k_scale=ks, v_scale=vs, partition_size=psize,
                             longest_context=longest, mean_context=mean)

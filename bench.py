@@ -349,9 +349,18 @@ def other_decode_configs(pa, torch, dev, launches, which=OTHER_CONFIGS):
         fns[name]()                                            # partials of this split
         torch.cuda.synchronize()
         merge_us[name] = round(time_in_graph(torch, merge, 20, 3, reps=32) * 1e3, 2)
+    graph_us = {}
+    if "cfg1" in which:
+        # config 1 is small enough for the host to set the pace of an eager call: the same launches
+        # replayed from a graph (device time; the launch policy then splits them, an eager call does not)
+        with pa.sizing_graph_workspace():
+            cfg1()
+        graph_us["cfg1"] = round(time_in_graph(torch, cfg1, 20, 3, reps=16) * 1e3, 2)
     for name, m in meta.items():
         us = med(t[name])
         rec = {"workload": m["workload"], "us": spread(t[name])}
+        if name in graph_us:
+            rec["us_in_replayed_graph"] = graph_us[name]
         if name in merge_us:
             rec["merge_pass_us_in_graph"] = merge_us[name]
         if "note" in m:

@@ -585,3 +585,32 @@ def test_matrix_kernel_in_a_replayed_graph(pa, gpu, cache):
         check(out1.cpu(), want, cache)
         check(out2.cpu(), want, cache)
         _ = torch.randn(1 << 16, device=gpu).sum().item()      # eager work between the replays
+
+
+def test_small_launches_are_split_for_graphs_and_not_for_eager_calls(pa, gpu):
+    """One row of 1000 tokens: replayed from a graph the launch policy cuts it into 64-token partitions (a
+    round of short workgroups), called eagerly it reads it in one pass (a second launch would cost the host
+    more than the split saves); a warm-up inside sizing_graph_workspace() is shaped like the capture that
+    follows, so the graphs' workspace is there when the capture needs it.  Same result every way."""
+    assert pa.choose_partition(1, 16, 8, 1008)[1] > 1 and pa.choose_partition(1, 16, 8, 1008, eager=True) == (0, 1)
+    c = cases.make_case(91, [1000], 80)
+    want = oracle_decode(c)
+    d = cases.to_device(c, gpu)
+    out = torch.empty_like(d["q"])
+    call = lambda: pa.paged_decode(d["q"], d["k_cache"], d["v_cache"], d["block_tables"], d["context_lens"], d["scale"], out=out)
+    call()
+    torch.cuda.synchronize()
+    check(out.cpu(), want, "fp16")
+    pa.release_decode_workspaces()
+    with pa.sizing_graph_workspace():
+        call()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    out.zero_()
+    with torch.cuda.graph(graph):
+        call()                                   # raises if the warm-up had not sized the graphs' workspace
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        check(out.cpu(), want, "fp16")

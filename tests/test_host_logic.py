@@ -100,6 +100,25 @@ def test_choose_partition_with_known_lengths(pa):
     assert cp(36, 16, 8, 8192, longest_context=0, mean_context=0) == cp(36, 16, 8, 8192)
 
 
+def test_choose_partition_for_eager_calls(pa):
+    """A launch issued call by call pays the host for the second launch of a split (a replayed graph
+    does not), so small launches stay one pass there and are split down to 64 tokens under replay."""
+    cp = pa.choose_partition
+    p, n = cp(1, 16, 8, 1008)
+    assert n > 1 and 64 <= p <= 128 and p % 16 == 0 and p * n >= 1008
+    assert cp(1, 16, 8, 1008, eager=True) == (0, 1)
+    assert cp(8, 16, 8, 512)[1] > 1 and cp(8, 16, 8, 512, eager=True) == (0, 1)
+    # a short row is one pass either way
+    assert cp(1, 16, 8, 256) == cp(1, 16, 8, 256, eager=True) == (0, 1)
+    # where the device time is beyond what two calls take to issue, the split stays; it may be coarser
+    # (every split below the host's pace costs the same), never finer
+    p_g, n_g = cp(1, 16, 8, 4096)
+    p_e, n_e = cp(1, 16, 8, 4096, eager=True)
+    assert 1 < n_e <= n_g and p_e * n_e >= 4096
+    assert cp(1, 16, 8, 32768, eager=True) == cp(1, 16, 8, 32768)
+    assert cp(64, 16, 8, 4096, eager=True) == (0, 1)
+
+
 def test_block_pool_layout(pa):
     pool = pa.BlockPool(4, 16, 2, 8, 128, dtype=torch.float16, device="cpu", cache_dtype="fp8")
     assert tuple(pool.kv_cache_tensor.shape) == (2, 2, 4, 16, 8, 128)
