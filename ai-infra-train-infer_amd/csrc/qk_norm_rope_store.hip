@@ -53,6 +53,10 @@ struct NormRopeParams {
 
 constexpr int kTokensPerGroup = 4;   // waves (= tokens) per workgroup
 constexpr int kMaxKvGroups = 4;      // K row groups a wave keeps in registers: kv_heads * head_dim <= 2048
+// Launches of up to this many tokens run one wave per (token, row group): 64 tokens 5.5 -> 3.7 us inside a
+// replayed graph, 512 tokens 6.0 -> 5.3; from 1024 tokens on the token-per-wave kernel is the faster one
+// (the angles are worked out once per token instead of once per row group).
+constexpr int64_t kSplitUpToTokens = 512;
 
 __device__ __forceinline__ float round_to_dtype(float x, int dtype) {
   if (dtype == PA_DTYPE_F16) return f16_bits_to_f32(f32_to_f16_bits(x));
@@ -256,6 +260,140 @@ __global__ __launch_bounds__(64 * kTokensPerGroup) void qk_norm_rope_store_kerne
   }
 }
 
+
+// The same work cut finer, for launches of few tokens (a decode step): one wave per (token, row
+// group) - a wave for each group of 64 / (head_dim / 8) query heads, one more for the token's K and V
+// rows (the fp8 writer's per-token amax runs over all K heads, so those stay in one wave).  A
+// decode step's 64 tokens then run as 320 short waves over 80 CUs instead of 64 long ones over 16,
+// and a wave's program is a sixth as long: straight-line code that runs once is fetched from
+// memory as it goes, which is most of what a launch of this size lasts.  Element for element the
+// arithmetic is the kernel's above.
+template <int D, bool FP8, int DT>
+__global__ __launch_bounds__(64 * kTokensPerGroup) void qk_norm_rope_store_split_kernel(const NormRopeParams p,
+                                                                                        const int q_groups) {
+  constexpr int LPR = D / 8;
+  constexpr int RPI = 64 / LPR;
+  constexpr int PAIR = LPR / 2;
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * kTokensPerGroup + (threadIdx.x >> 6);
+  const int roles = q_groups + 1;
+  const int64_t t = w / roles;
+  const int role = __builtin_amdgcn_readfirstlane((int)(w % roles));   // < q_groups: that group of q rows; else K and V
+  if (t >= p.num_tokens) return;      // the whole wave
+  const int c = lane % LPR;
+  const int sub = lane / LPR;
+  const bool upper = c >= PAIR;
+  const int f0 = (c % PAIR) * 8;
+  const bool is_q = role < q_groups;
+
+  const float pos = (float)p.positions[t];
+  const float4 fa = *(const float4*)(p.inv_freq + f0), fb = *(const float4*)(p.inv_freq + f0 + 4);
+  float wt[8], x[kMaxKvGroups][8], vx[kMaxKvGroups][8];
+#pragma unroll
+  for (int g = 0; g < kMaxKvGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[g][e] = vx[g][e] = 0.0f;
+  const bool write = p.k_cache != nullptr;
+  int64_t slot = -1;
+  if (is_q) {
+    load8_as_f32(p.q_weight, c * 8, p.weight_dtype, wt);
+    const int head = role * RPI + sub;
+    if (head < p.hq) load8_as_f32(p.q, t * p.q_stride + (int64_t)head * D + c * 8, DT, x[0]);
+  } else {
+    load8_as_f32(p.k_weight, c * 8, p.weight_dtype, wt);
+    if (write) slot = (int64_t)p.slot_mapping[t];
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) {
+        load8_as_f32(p.k, t * p.k_stride + (int64_t)head * D + c * 8, DT, x[g]);
+        if (write) load8_as_f32(p.v, t * p.v_stride + (int64_t)head * D + c * 8, DT, vx[g]);
+      }
+    }
+  }
+
+  float cs[8], sn[8];
+  {
+    const float fr[8] = {fa.x, fa.y, fa.z, fa.w, fb.x, fb.y, fb.z, fb.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sincos_turns(pos * fr[e], sn[e], cs[e]);
+  }
+
+  // one row group: the loop below runs once for a q wave, once per K row group for the other
+  const int groups = is_q ? 1 : (p.hkv + RPI - 1) / RPI;
+#pragma unroll
+  for (int g = 0; g < kMaxKvGroups; ++g) {
+    if (g >= groups) continue;         // wave-uniform
+    float (&r)[8] = x[g];
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += r[e] * r[e];
+    ss += dpp_f32<0xB1>(ss);
+    ss += dpp_f32<0x4E>(ss);
+    if constexpr (LPR == 16) {
+      ss += dpp_f32<0x124>(ss);
+      ss += dpp_f32<0x128>(ss);
+    } else {
+      ss += dpp_f32<0x141>(ss);
+    }
+    const float inv = rsqrtf(ss / (float)D + p.eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float y = round_to_dtype(wt[e] * (r[e] * inv), DT);
+      const float other = LPR == 16 ? dpp_f32<0x128>(y) : __shfl_xor(y, PAIR);
+      const float rotated = upper ? other : -other;
+      r[e] = round_to_dtype(y * cs[e] + rotated * sn[e], DT);
+    }
+  }
+
+  if (is_q) {
+    const int head = role * RPI + sub;
+    if (head < p.hq) store8_from_f32(p.q_out, t * p.q_out_stride + (int64_t)head * D + c * 8, DT, x[0]);
+    return;
+  }
+  if (p.k_out) {
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) store8_from_f32(p.k_out, t * p.k_out_stride + (int64_t)head * D + c * 8, DT, x[g]);
+    }
+  }
+  if (!write || slot < 0 || slot >= p.total_slots) return;   // uniform over the wave
+  const int64_t row = (int64_t)p.hkv * D;
+  if constexpr (!FP8) {
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) {
+        store8_from_f32(p.k_cache, slot * row + (int64_t)head * D + c * 8, DT, x[g]);
+        store8_from_f32(p.v_cache, slot * row + (int64_t)head * D + c * 8, DT, vx[g]);
+      }
+    }
+  } else {
+    float ka = 0.0f, va = 0.0f;
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ka = nan_keeping_max(ka, fabsf(x[g][e]));
+        va = nan_keeping_max(va, fabsf(vx[g][e]));
+      }
+    const float ksc = wave_scale(ka), vsc = wave_scale(va);
+    if (lane == 0) {
+      p.k_scale[slot] = ksc;
+      p.v_scale[slot] = vsc;
+    }
+#pragma unroll
+    for (int g = 0; g < kMaxKvGroups; ++g) {
+      const int head = g * RPI + sub;
+      if (head < p.hkv) {
+        *(uint2*)(p.k_cache + slot * row + (int64_t)head * D + c * 8) = encode8(x[g], ksc);
+        *(uint2*)(p.v_cache + slot * row + (int64_t)head * D + c * 8) = encode8(vx[g], vsc);
+      }
+    }
+  }
+}
+
 }  // namespace pa
 
 using namespace pa;
@@ -322,8 +460,17 @@ extern "C" int pa_qk_norm_rope_store(const void* q, const void* k, const void* v
 
   dim3 grid((unsigned)((num_tokens + kTokensPerGroup - 1) / kTokensPerGroup));
   hipStream_t st = (hipStream_t)stream;
-#define PA_LAUNCH_NORM_ROPE(DIM, F8, DT) \
-  hipLaunchKernelGGL((qk_norm_rope_store_kernel<DIM, F8, DT>), grid, dim3(64 * kTokensPerGroup), 0, st, p)
+  // few tokens: one wave per (token, row group) instead of one per token
+  const int rows_per_wave = 64 / ((int)head_dim / 8);
+  const int q_groups = ((int)num_q_heads + rows_per_wave - 1) / rows_per_wave;
+  const bool split = num_tokens <= kSplitUpToTokens;
+  if (split) grid = dim3((unsigned)((num_tokens * (q_groups + 1) + kTokensPerGroup - 1) / kTokensPerGroup));
+#define PA_LAUNCH_NORM_ROPE(DIM, F8, DT)                                                                         \
+  if (split)                                                                                                     \
+    hipLaunchKernelGGL((qk_norm_rope_store_split_kernel<DIM, F8, DT>), grid, dim3(64 * kTokensPerGroup), 0, st, p, \
+                       q_groups);                                                                                \
+  else                                                                                                           \
+    hipLaunchKernelGGL((qk_norm_rope_store_kernel<DIM, F8, DT>), grid, dim3(64 * kTokensPerGroup), 0, st, p)
 #define PA_LAUNCH_NORM_ROPE_DT(DIM, F8)                                  \
   switch (dtype) {                                                       \
     case PA_DTYPE_F16: PA_LAUNCH_NORM_ROPE(DIM, F8, PA_DTYPE_F16); break;   \

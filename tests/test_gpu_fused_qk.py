@@ -36,7 +36,7 @@ def run(pa, c, gpu, **kw):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("t,hq,hkv,d", [(64, 16, 8, 128), (5, 8, 8, 128), (33, 8, 2, 64), (1, 4, 4, 64)])
+@pytest.mark.parametrize("t,hq,hkv,d", [(64, 16, 8, 128), (5, 8, 8, 128), (33, 8, 2, 64), (1, 4, 4, 64), (600, 16, 8, 128), (515, 4, 2, 64)])
 def test_values_against_the_oracle(pa, gpu, dtype, t, hq, hkv, d):
     c = make(70 + t + d, t, hq, hkv, d, dtype)
     q_out, k_out = run(pa, c, gpu, return_k=True)
@@ -99,6 +99,45 @@ def test_fp8_cache_write_equals_the_separate_quantising_store(pa, gpu, hkv, d):
     b = lambda x: x.view(torch.uint8).cpu()
     assert torch.equal(b(kc), b(kc2)) and torch.equal(b(vc), b(vc2))
     assert torch.equal(ks.cpu(), ks2.cpu()) and torch.equal(vs.cpu(), vs2.cpu())
+
+
+@pytest.mark.parametrize("cache", ["fp16", "fp8"])
+@pytest.mark.parametrize("hq,hkv,d", [(16, 8, 128), (6, 2, 64)])
+def test_both_launch_shapes_write_the_same_bytes(pa, gpu, cache, hq, hkv, d):
+    """Launches of up to 512 tokens run one wave per (token, row group), longer ones one wave per token:
+    a chunk of 640 tokens and its two halves must produce the same q, K and cache bytes."""
+    t, bs = 640, 16
+    nb = t // bs + 3
+    c = make(75, t, hq, hkv, d, torch.float16)
+    c["k"][17] = 0.0
+    slots = torch.randperm(nb * bs, generator=torch.Generator().manual_seed(8))[:t].to(torch.int32)
+    slots[5] = -1
+    slots[400] = -1
+    dev = lambda x: x.to(gpu)
+
+    def pool():
+        if cache == "fp8":
+            z = lambda: torch.zeros(nb, bs, hkv, d, dtype=torch.float8_e4m3fn, device=gpu)
+            return dict(k_cache=z(), v_cache=z(), k_scale=torch.ones(nb, bs, device=gpu), v_scale=torch.ones(nb, bs, device=gpu),
+                        cache_dtype="fp8")
+        z = lambda: torch.full((nb, bs, hkv, d), 3.0, dtype=torch.float16, device=gpu)
+        return dict(k_cache=z(), v_cache=z())
+
+    def call(lo, hi, kw):
+        return pa.qk_norm_rope_store(dev(c["q"][lo:hi]), dev(c["k"][lo:hi]), dev(c["v"][lo:hi]), dev(c["qw"]), dev(c["kw"]),
+                                     c["eps"], dev(c["inv_freq"]), dev(c["pos"][lo:hi]), slot_mapping=dev(slots[lo:hi]),
+                                     return_k=True, **kw)
+
+    whole, halves = pool(), pool()
+    q1, k1 = call(0, t, whole)
+    parts = [call(0, t // 2, halves), call(t // 2, t, halves)]
+    torch.cuda.synchronize()
+    assert torch.equal(q1, torch.cat([p[0] for p in parts])) and torch.equal(k1, torch.cat([p[1] for p in parts]))
+    for name in whole:
+        if name != "cache_dtype":
+            a, b = whole[name], halves[name]
+            assert torch.equal(a.view(torch.uint8) if a.dtype == torch.float8_e4m3fn else a,
+                               b.view(torch.uint8) if b.dtype == torch.float8_e4m3fn else b), name
 
 
 def test_packed_qkv_views_and_errors(pa, lib, gpu):
