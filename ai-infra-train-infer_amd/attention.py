@@ -46,8 +46,18 @@ def _require_gpu(t, what):
             "package has no CPU path" % (what, t.device))
 
 
+# The current stream's handle without building a torch.cuda.Stream object around it: this runs once per
+# kernel launch, and an eager decode step makes 140 of them.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(device):
-    return torch.cuda.current_stream(device).cuda_stream
+    idx = device if isinstance(device, int) else device.index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    if _raw_stream is not None:
+        return _raw_stream(idx)
+    return torch.cuda.current_stream(idx).cuda_stream
 
 
 def _rows(t, what):
@@ -189,7 +199,8 @@ def qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, eps, inv_freq, pos
         raise RuntimeError("qk_norm_rope_store: inv_freq must be fp32 [head_dim / 2]")
     if positions.numel() != n:
         raise RuntimeError("qk_norm_rope_store: positions has %d entries for %d tokens" % (positions.numel(), n))
-    positions = positions.to(torch.int64).contiguous()
+    if positions.dtype != torch.int64 or not positions.is_contiguous():
+        positions = positions.to(torch.int64).contiguous()
     q_out = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
     k_out = torch.empty((n, hkv, d), dtype=q.dtype, device=q.device) if return_k else None
     write = k_cache is not None and slot_mapping is not None
@@ -304,7 +315,8 @@ def add_rms_norm(x, weight, eps=1e-6, delta=None, inplace_sum=True):
     _require_gpu(x, "add_rms_norm")
     lib = _native.load()
     shape = x.shape
-    x2, xs = _rows2d(x.reshape(-1, shape[-1]), "add_rms_norm")
+    flat = len(shape) == 2          # the decoder block's own call: nothing to reshape on the way in or out
+    x2, xs = _rows2d(x if flat else x.reshape(-1, shape[-1]), "add_rms_norm")
     rows, hidden = x2.shape
     code = _code(x2.dtype, "add_rms_norm")
     normed = torch.empty((rows, hidden), dtype=x2.dtype, device=x2.device)
@@ -315,7 +327,7 @@ def add_rms_norm(x, weight, eps=1e-6, delta=None, inplace_sum=True):
     if delta is not None:
         if delta.shape != shape or delta.dtype != x.dtype:
             raise RuntimeError("add_rms_norm: delta must match x in shape and dtype")
-        d2, ds = _rows2d(delta.reshape(-1, hidden), "add_rms_norm")
+        d2, ds = _rows2d(delta if flat else delta.reshape(-1, hidden), "add_rms_norm")
         total = x2 if inplace_sum else torch.empty((rows, hidden), dtype=x2.dtype, device=x2.device)
     rc = lib.pa_add_rms_norm(x2.data_ptr(), xs, d2.data_ptr() if d2 is not None else None, ds or 0,
                              weight.data_ptr(), _code(weight.dtype, "add_rms_norm"), float(eps),
@@ -323,6 +335,8 @@ def add_rms_norm(x, weight, eps=1e-6, delta=None, inplace_sum=True):
                              (total.stride(0) if rows > 1 else hidden) if d2 is not None else 0,
                              normed.data_ptr(), hidden, code, rows, hidden, _stream_ptr(x2.device))
     _native.check(rc, "pa_add_rms_norm")
+    if flat:
+        return total, normed
     return total.view(shape), normed.view(shape)
 
 
@@ -466,10 +480,10 @@ def reserve_decode_workspace(device, nbytes, for_graphs=False):
     inside sizing_graph_workspace() do it too); inside a capture a workspace that is too small
     raises instead of allocating from the graph's pool."""
     idx = _device_index(device)
-    capturing = torch.cuda.is_current_stream_capturing()
+    capturing = _is_capturing()
     if _sizing_for_graphs and not capturing and not for_graphs:
         reserve_decode_workspace(device, nbytes, for_graphs=True)
-    key = (idx, _GRAPHS if (for_graphs or capturing) else torch.cuda.current_stream(idx).cuda_stream)
+    key = (idx, _GRAPHS if (for_graphs or capturing) else _stream_ptr(idx))
     held = _WORKSPACES.setdefault(key, [])
     if held and held[-1].numel() >= nbytes:
         return held[-1]
