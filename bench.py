@@ -1004,7 +1004,7 @@ def main():
     ap.add_argument("--sections", default="all",
                     help="comma-separated parts to run: headline (the FP16 / FP8 launches), probe (the same "
                          "launches with loads only), others (configs 1, 3, 4), ragged (rows of unequal length under wide tables), gqa (wider query groups), prefill, "
-                         "extras, cpu, stores (the KV-cache write alone; also part of extras); 'all' = every one.  For profiler runs, which want one kind of launch "
+                         "extras, cpu, stores (the KV-cache write alone; also part of extras), model (the 28-layer decode step alone; also part of extras); 'all' = every one.  For profiler runs, which want one kind of launch "
                          "per kernel name: the load probe is the decode kernel itself with a flag set, and the "
                          "other configurations launch the headline's kernels on other shapes.  Without "
                          "`headline` the run prints a reduced line for the parts it ran")
@@ -1032,7 +1032,7 @@ def main():
         sections.discard("extras")
     if args.no_cpu_baseline:
         sections.discard("cpu")
-    unknown = sections - {"headline", "probe", "others", "ragged", "gqa", "prefill", "extras", "cpu", "stores"}
+    unknown = sections - {"headline", "probe", "others", "ragged", "gqa", "prefill", "extras", "cpu", "stores", "model"}
     if unknown:
         print("bench.py: unknown section(s) %s" % sorted(unknown), file=sys.stderr)
         sys.exit(2)
@@ -1057,6 +1057,8 @@ def main():
         if "stores" in sections:
             part["kv_store"] = kv_store_times(pa, torch, dev, args.steps, args.warmup,
                                               [int(x) for x in args.store_tokens.split(",")])
+        if "model" in sections:
+            part["model_decode_step"] = model_step_cfg5b(pa, torch, dev, min(args.steps, 20), min(args.warmup, 10))
         print(json.dumps(part))
         return
     probe_only = "headline" not in sections and "cpu" not in sections
