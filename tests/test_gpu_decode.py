@@ -86,7 +86,7 @@ def test_query_group_layouts_keep_the_result(pa, gpu, hq, hkv, qpw, cache):
     check(gpu_decode(pa, c, gpu, q_heads_per_wave=qpw, waves=4), want, cache)
 
 
-@pytest.mark.parametrize("bs", [8, 32, 128])
+@pytest.mark.parametrize("bs", [8, 32, 128, 256])
 @pytest.mark.parametrize("cache", ["fp16", "fp8"])
 def test_block_sizes(pa, gpu, bs, cache):
     lens = [1, bs - 1, bs, bs + 1, 5 * bs + 3, 301]
@@ -463,7 +463,7 @@ def test_matrix_kernel_head_shapes(pa, gpu, hq, hkv, d, cache):
         check(gpu_decode(pa, c, gpu, q_heads_per_wave=16, **kw), want, cache)
 
 
-@pytest.mark.parametrize("bs", [8, 32, 128])
+@pytest.mark.parametrize("bs", [8, 32, 128, 256])
 @pytest.mark.parametrize("cache", ["fp16", "fp8"])
 def test_matrix_kernel_block_sizes_and_empty_rows(pa, gpu, bs, cache):
     lens = [1, 0, bs - 1, bs, bs + 1, 5 * bs + 3, 0, 301]

@@ -109,7 +109,7 @@ def test_head_shapes(pa, gpu, hq, hkv, d, waves):
     check(gpu_prefill(pa, c, gpu, waves), oracle_prefill(c, upcast=True))
 
 
-@pytest.mark.parametrize("bs", [8, 32])
+@pytest.mark.parametrize("bs", [8, 32, 256])
 def test_block_sizes(pa, gpu, bs, waves):
     c = make_prefill(62, [bs * 3 + 1, 0], [100, 77], 64, block_size=bs)
     check(gpu_prefill(pa, c, gpu, waves), oracle_prefill(c, upcast=True))
