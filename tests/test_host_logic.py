@@ -119,6 +119,26 @@ def test_choose_partition_for_eager_calls(pa):
     assert cp(64, 16, 8, 4096, eager=True) == (0, 1)
 
 
+def test_choose_partition_invariants_over_random_shapes(pa):
+    """Whatever the shape and the hints: one pass, or partitions of a multiple of 16 tokens (64 at least),
+    no more than the limit, that cover the bound with none to spare."""
+    import random
+    rnd = random.Random(1)
+    cp, kl = pa.choose_partition, pa.attention._known_lengths
+    for _ in range(5000):
+        batch = rnd.choice([1, 2, 3, 4, 7, 8, 16, 31, 32, 36, 64, 100, 128, 256, 1000])
+        hkv = rnd.choice([1, 2, 4, 8])
+        hq = hkv * rnd.choice([1, 2, 3, 4, 8, 16])
+        ctx = rnd.choice([16, 48, 64, 256, 512, 1008, 1024, 2048, 4096, 8192, 32768, 131072, 16 * rnd.randint(1, 9000)])
+        longest = rnd.choice([None, 0, rnd.randint(1, 2 * ctx)])
+        mean = rnd.choice([None, 0, rnd.random() * ctx])
+        args = (batch, hq, hkv, ctx, rnd.choice([64, 128]), rnd.choice([1, 2]), rnd.choice([256, 304, 64]), longest, mean,
+                rnd.choice([False, True]))
+        p, n = cp(*args)
+        bound = kl(ctx, longest, mean)[0]
+        assert (p, n) == (0, 1) or (p % 16 == 0 and p >= 64 and 2 <= n <= 129 and p * (n - 1) < bound <= p * n), (args, p, n)
+
+
 def test_block_pool_layout(pa):
     pool = pa.BlockPool(4, 16, 2, 8, 128, dtype=torch.float16, device="cpu", cache_dtype="fp8")
     assert tuple(pool.kv_cache_tensor.shape) == (2, 2, 4, 16, 8, 128)
