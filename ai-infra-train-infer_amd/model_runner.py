@@ -402,6 +402,12 @@ class ModelRunner:
         self._hf_model: Optional[torch.nn.Module] = None
         self._state_graph_lookup: Dict[tuple, object] = {}
         self._prefix_groups_kept = None          # (signature of the batch, PrefixGroups or None) of the last decode step
+        # pinned staging buffers for prepare_decode's upload, used in turn; an event marks when the copy
+        # out of one is done.  (A fresh pinned tensor per step comes out of torch's caching host
+        # allocator, which hands a block out again only after its copy has run: a host that prepares
+        # steps faster than the GPU takes them makes it allocate a new block every step.)
+        self._decode_stage = [[None, None] for _ in range(4)]
+        self._decode_stage_turn = 0
         # how run_decode_state ran its steps: replays of a graph recorded over the shared-prefix launch,
         # replays of a plain graph, eager forwards
         self.decode_state_stats = {"shared_prefix_graph": 0, "plain_graph": 0, "ragged_graph": 0, "eager": 0}
@@ -604,7 +610,14 @@ class ModelRunner:
         o_slots = o_pos + pad(8 * n)
         o_lens = o_slots + pad(4 * n)
         o_tables = o_lens + pad(4 * n)
-        stage = np.empty(o_tables + 4 * n * width, np.uint8)
+        nbytes = o_tables + 4 * n * width
+        slot = self._decode_stage[self._decode_stage_turn]
+        self._decode_stage_turn = (self._decode_stage_turn + 1) % len(self._decode_stage)
+        if slot[1] is not None:
+            slot[1].synchronize()          # the copy out of this buffer, four steps ago
+        if slot[0] is None or slot[0].numel() < nbytes:
+            slot[0] = torch.empty(max(2 * nbytes, 1 << 16), dtype=torch.uint8).pin_memory()
+        stage = slot[0].numpy()[:nbytes]
         stage[0:8 * n].view(np.int64)[:] = ids
         stage[o_pos:o_pos + 8 * n].view(np.int64)[:] = pos
         stage[o_slots:o_slots + 4 * n].view(np.int32)[:] = slots
@@ -614,7 +627,11 @@ class ModelRunner:
         for i, bt in enumerate(lists):
             if len(bt):
                 tables[i, :len(bt)] = bt
-        dev = torch.from_numpy(stage).pin_memory().to(self._device(), non_blocking=True)
+        dev = torch.empty(nbytes, dtype=torch.uint8, device=self._device())
+        dev.copy_(slot[0][:nbytes], non_blocking=True)
+        if slot[1] is None:
+            slot[1] = torch.cuda.Event()
+        slot[1].record()
         set_context(
             is_prefill=False,
             slot_mapping=dev[o_slots:o_slots + 4 * n].view(torch.int32),
