@@ -10,8 +10,8 @@ same context out (int32 `slot_mapping`, `context_lens`, `cu_seqlens_*`, `block_t
 
   * the reference builds the block table with one Python assignment per entry
     (`tables[i, j] = block_id`, 16 384 device writes at batch 64 / ctx 4096) and a fresh
-    torch.tensor(...) per field; here every field is built with numpy row copies and shipped
-    from pinned memory with one asynchronous copy per field;
+    torch.tensor(...) per field; here the fields of a step are built with numpy row copies side by
+    side in one pinned staging buffer and shipped with one asynchronous copy;
   * graph replay copies into static device buffers and pads with slot -1 / context 0, exactly as
     the reference does, but capture needs no host synchronisation inside the model;
   * `run_batch_decode` gets its slot mapping from a kernel instead of two `.item()` reads per
