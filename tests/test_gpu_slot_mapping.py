@@ -266,3 +266,34 @@ def test_prefill_chunks_take_their_tables_from_the_decode_state(pa, gpu):
     with pytest.raises(RuntimeError, match="not a reserved row"):
         st.activate(1, 10, 3)
     pa.reset_context()
+
+
+def test_prepare_decode_on_the_device_equals_the_reference_loops(pa, gpu):
+    """ModelRunner.prepare_decode on the GPU: the five fields go up side by side through a ring of pinned
+    staging buffers as one copy - every field equal to the reference's host loops, over more steps
+    than the ring has buffers, batches that grow past a buffer's size, and while earlier steps' tensors
+    are still held (a later step must not overwrite what an earlier one handed out)."""
+    import random
+    from test_model_runner_host import random_sequences, as_list
+    rng = random.Random(21)
+    runner = pa.ModelRunner(None, pa.ModelRunnerConfig(block_size=16, device="cuda:0"))
+    held = []
+    for trial in range(11):
+        n = rng.randint(1, 12) if trial < 8 else 300 * (trial - 7)        # then 300, 600, 900 rows
+        seqs = random_sequences(rng, n, 16, prefill=False)
+        if trial == 0:
+            seqs[0]["last_block_num_tokens"] = 3
+        ids, pos = runner.prepare_decode(seqs)
+        ctx = pa.get_context()
+        want = mro.decode_metadata(seqs, 16)
+        held.append((ids, pos, ctx.slot_mapping, ctx.context_lens, ctx.block_tables, want))
+        assert ids.is_cuda and ids.dtype == torch.long and pos.dtype == torch.long
+        for t in (ctx.slot_mapping, ctx.context_lens, ctx.block_tables):
+            assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous() and t.data_ptr() % 16 == 0
+        assert ctx.longest_context_len == max(want["context_lens"])
+    torch.cuda.synchronize()
+    for ids, pos, slots, lens, tables, want in held:
+        assert ids.tolist() == want["input_ids"] and pos.tolist() == want["positions"]
+        assert as_list(slots) == want["slot_mapping"] and as_list(lens) == want["context_lens"]
+        assert as_list(tables) == want["block_tables"]
+    pa.reset_context()
