@@ -402,7 +402,7 @@ class ModelRunner:
         self._hf_model: Optional[torch.nn.Module] = None
         self._state_graph_lookup: Dict[tuple, object] = {}
         self._prefix_groups_kept = None          # (signature of the batch, PrefixGroups or None) of the last decode step
-        # pinned staging buffers for prepare_decode's upload, used in turn; an event marks when the copy
+        # pinned staging buffers for the uploads of prepare_decode and prepare_prefill, used in turn; an event marks when the copy
         # out of one is done.  (A fresh pinned tensor per step comes out of torch's caching host
         # allocator, which hands a block out again only after its copy has run: a host that prepares
         # steps faster than the GPU takes them makes it allocate a new block every step.)
@@ -448,6 +448,27 @@ class ModelRunner:
             return t
         return t.pin_memory().to(dev, non_blocking=True)
 
+    def _staging(self, nbytes):
+        """The next pinned staging buffer of the ring, at least nbytes long (uint8), and its ring slot;
+        _upload(slot, nbytes) ships its first nbytes.  Waits for the copy that last left the buffer
+        (as many steps ago as the ring has buffers)."""
+        slot = self._decode_stage[self._decode_stage_turn]
+        self._decode_stage_turn = (self._decode_stage_turn + 1) % len(self._decode_stage)
+        if slot[1] is not None:
+            slot[1].synchronize()
+        if slot[0] is None or slot[0].numel() < nbytes:
+            slot[0] = torch.empty(max(2 * nbytes, 1 << 16), dtype=torch.uint8).pin_memory()
+        return slot[0][:nbytes], slot
+
+    def _upload(self, slot, nbytes):
+        """One asynchronous copy of the staging buffer's first nbytes to a fresh device tensor."""
+        dev = torch.empty(nbytes, dtype=torch.uint8, device=self._device())
+        dev.copy_(slot[0][:nbytes], non_blocking=True)
+        if slot[1] is None:
+            slot[1] = torch.cuda.Event()
+        slot[1].record()
+        return dev
+
     def _prepare_block_tables(self, sequences, device=None):
         """[num_seqs, max_blocks] int32, padded with -1; None when no sequence has a table."""
         lists = [seq.get("block_table", []) for seq in sequences]
@@ -488,7 +509,7 @@ class ModelRunner:
         width = 0 if from_state or not any_table else max(len(bt) for bt in lists)
         # one pinned staging buffer: ids int64 [total] | cu_q int32 [S+1] | cu_k int32 [S+1] | rows int32 [S] | tables int32 [S, width]
         n32 = 2 * (S + 1) + S + S * width
-        stage = torch.empty(8 * total + 4 * n32, dtype=torch.uint8).pin_memory()
+        stage, slot = self._staging(8 * total + 4 * n32)
         ids = stage[:8 * total].view(torch.long)
         meta = stage[8 * total:].view(torch.int32)
         ids_np, meta_np = ids.numpy(), meta.numpy()
@@ -509,7 +530,7 @@ class ModelRunner:
             rows_np[i] = seq["state_row"] if from_state else i
             if tables_np is not None and len(lists[i]):
                 tables_np[i, :len(lists[i])] = lists[i]
-        on_dev = stage.to(dev, non_blocking=True)
+        on_dev = self._upload(slot, 8 * total + 4 * n32)
         input_ids = on_dev[:8 * total].view(torch.long)
         meta_dev = on_dev[8 * total:].view(torch.int32)
         cu_q_dev, cu_k_dev = meta_dev[:S + 1], meta_dev[S + 1:2 * (S + 1)]
@@ -611,13 +632,8 @@ class ModelRunner:
         o_lens = o_slots + pad(4 * n)
         o_tables = o_lens + pad(4 * n)
         nbytes = o_tables + 4 * n * width
-        slot = self._decode_stage[self._decode_stage_turn]
-        self._decode_stage_turn = (self._decode_stage_turn + 1) % len(self._decode_stage)
-        if slot[1] is not None:
-            slot[1].synchronize()          # the copy out of this buffer, four steps ago
-        if slot[0] is None or slot[0].numel() < nbytes:
-            slot[0] = torch.empty(max(2 * nbytes, 1 << 16), dtype=torch.uint8).pin_memory()
-        stage = slot[0].numpy()[:nbytes]
+        pinned, slot = self._staging(nbytes)
+        stage = pinned.numpy()
         stage[0:8 * n].view(np.int64)[:] = ids
         stage[o_pos:o_pos + 8 * n].view(np.int64)[:] = pos
         stage[o_slots:o_slots + 4 * n].view(np.int32)[:] = slots
@@ -627,11 +643,7 @@ class ModelRunner:
         for i, bt in enumerate(lists):
             if len(bt):
                 tables[i, :len(bt)] = bt
-        dev = torch.empty(nbytes, dtype=torch.uint8, device=self._device())
-        dev.copy_(slot[0][:nbytes], non_blocking=True)
-        if slot[1] is None:
-            slot[1] = torch.cuda.Event()
-        slot[1].record()
+        dev = self._upload(slot, nbytes)
         set_context(
             is_prefill=False,
             slot_mapping=dev[o_slots:o_slots + 4 * n].view(torch.int32),
