@@ -407,6 +407,7 @@ class ModelRunner:
         # allocator, which hands a block out again only after its copy has run: a host that prepares
         # steps faster than the GPU takes them makes it allocate a new block every step.)
         self._decode_stage = [[None, None] for _ in range(4)]
+        self._table_rows = {}          # prepare_decode: (length, first id, last id) -> (copy of the block-id list, int32 row)
         self._decode_stage_turn = 0
         # how run_decode_state ran its steps: replays of a graph recorded over the shared-prefix launch,
         # replays of a plain graph, eager forwards
@@ -588,20 +589,21 @@ class ModelRunner:
         """sequences: dicts with 'token_ids', 'block_table', optional 'last_block_num_tokens'.
         One token per sequence; context_lens counts the token being written."""
         n = len(sequences)
-        ids = np.empty(n, np.int64)
-        pos = np.empty(n, np.int64)
-        slots = np.empty(n, np.int32)
-        lens = np.empty(n, np.int32)
-        for i, seq in enumerate(sequences):
+        bs = self.block_size
+        ids_l, lens_l, slots_l = [], [], []
+        for seq in sequences:
             toks = seq["token_ids"]
-            position = len(toks) - 1
+            length = len(toks)
             last = seq.get("last_block_num_tokens", None)
             if last is None:
-                last = (position % self.block_size) + 1
-            ids[i] = toks[-1]
-            pos[i] = position
-            slots[i] = seq["block_table"][-1] * self.block_size + last - 1
-            lens[i] = len(toks)
+                last = ((length - 1) % bs) + 1
+            ids_l.append(toks[-1])
+            lens_l.append(length)
+            slots_l.append(seq["block_table"][-1] * bs + last - 1)
+        ids = np.array(ids_l, np.int64)
+        lens = np.array(lens_l, np.int32)
+        pos = lens.astype(np.int64) - 1
+        slots = np.array(slots_l, np.int32)
         groups = None
         if getattr(self.config, "share_prefix_decode", False) and self._device() != "cpu":
             groups = self._decode_prefix_groups([seq["block_table"] for seq in sequences], lens.tolist())
@@ -640,9 +642,26 @@ class ModelRunner:
         stage[o_lens:o_lens + 4 * n].view(np.int32)[:] = lens
         tables = stage[o_tables:].view(np.int32).reshape(n, width)
         tables.fill(-1)
+        # Turning a sequence's Python list of block ids into int32 costs more than everything else in
+        # this function (8192 integers at batch 64 x ctx 2048), and the lists change once in block_size
+        # steps.  The rows of the last step are kept, found again by (length, first id, last id) and
+        # reused only when the kept copy of the list still equals the caller's list (a comparison at
+        # C speed); whatever else changed - an appended block, a copied-on-write block, a new
+        # sequence in the slot - is converted afresh.
+        kept, fresh = self._table_rows, {}
         for i, bt in enumerate(lists):
-            if len(bt):
-                tables[i, :len(bt)] = bt
+            length = len(bt)
+            if length:
+                if type(bt) is list:
+                    key = (length, bt[0], bt[-1])
+                    hit = kept.get(key)
+                    if hit is None or hit[0] != bt:
+                        hit = (list(bt), np.asarray(bt, dtype=np.int32))
+                    fresh[key] = hit
+                    tables[i, :length] = hit[1]
+                else:
+                    tables[i, :length] = bt
+        self._table_rows = fresh
         dev = self._upload(slot, nbytes)
         set_context(
             is_prefill=False,

@@ -296,4 +296,27 @@ def test_prepare_decode_on_the_device_equals_the_reference_loops(pa, gpu):
         assert ids.tolist() == want["input_ids"] and pos.tolist() == want["positions"]
         assert as_list(slots) == want["slot_mapping"] and as_list(lens) == want["context_lens"]
         assert as_list(tables) == want["block_tables"]
+    # The converted rows of a step are kept for the next one: whatever a caller does to a list between two
+    # steps must show - a block appended, the last block replaced (copy-on-write), a block in the middle
+    # replaced in place (same length, same first and last id), a list swapped for another, a tuple.
+    seqs = [{"token_ids": [7] * (16 * 5 + 3), "block_table": [10 * i + j for j in range(6)]} for i in range(1, 7)]
+
+    def check():
+        runner.prepare_decode(seqs)
+        ctx = pa.get_context()
+        want = mro.decode_metadata(seqs, 16)
+        assert as_list(ctx.block_tables) == want["block_tables"] and as_list(ctx.slot_mapping) == want["slot_mapping"]
+
+    check()
+    check()
+    seqs[0]["block_table"].append(777)
+    seqs[0]["token_ids"] += [7] * 16
+    seqs[1]["block_table"][-1] = 888
+    seqs[2]["block_table"][2] = 999
+    seqs[3]["block_table"] = list(seqs[4]["block_table"])
+    seqs[5]["block_table"] = tuple(seqs[5]["block_table"])
+    check()
+    seqs[2]["block_table"][2] = 22
+    seqs.reverse()
+    check()
     pa.reset_context()
