@@ -66,6 +66,45 @@ SIGNATURES = {
     "pa_check_tables": (_int, [_ptr, _i64, _i64, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
 }
 
+# Entry points a decode step calls once or more per layer: bound through pa_fastcall (a small CPython
+# module, csrc/fastcall) when it has been built, because ctypes spends 3-5 us converting their 10-35
+# arguments and the module 0.3 us.  Their callers pass addresses and sizes as plain ints, None for a
+# null pointer and floats for floats, which is all the module accepts; every other entry, and every
+# entry when the module is missing, goes through ctypes.
+FAST_ENTRIES = ("pa_decode", "pa_decode_shared_prefix", "pa_qk_norm_rope_store", "pa_add_rms_norm", "pa_silu_mul",
+                "pa_kv_store", "pa_kv_store_fp8", "pa_prefill", "pa_sample")
+_KIND = {_ptr: "p", _i64: "q", _int: "i", _f32: "f"}
+
+
+class _Library:
+    """The loaded library.  Attributes are its entry points: ctypes functions, or pa_fastcall bindings of
+    the same addresses with the same arguments and return values."""
+
+    def __init__(self, cdll, fast):
+        self._cdll = cdll
+        self.fast_entries = tuple(sorted(fast))
+        for name in SIGNATURES:
+            setattr(self, name, fast.get(name) or getattr(cdll, name))
+
+    def __getattr__(self, name):          # entry points outside SIGNATURES (none today) and dunder lookups
+        return getattr(self._cdll, name)
+
+
+def _fast_bindings(cdll):
+    try:
+        from . import pa_fastcall
+    except ImportError:
+        return {}
+    import functools
+    fast = {}
+    for name in FAST_ENTRIES:
+        restype, argtypes = SIGNATURES[name]
+        addr = ctypes.cast(getattr(cdll, name), ctypes.c_void_p).value
+        index = pa_fastcall.bind(addr, "".join(_KIND[t] for t in argtypes), restype is _i64)
+        fast[name] = functools.partial(pa_fastcall.call, index)
+    return fast
+
+
 _lock = threading.Lock()
 _lib = None
 
@@ -95,7 +134,7 @@ def load():
             fn = getattr(lib, name)
             fn.restype = restype
             fn.argtypes = argtypes
-        _lib = lib
+        _lib = _Library(lib, _fast_bindings(lib))
     return _lib
 
 

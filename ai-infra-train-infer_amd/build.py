@@ -115,7 +115,32 @@ def build_library(force=True, verbose=False):
         if r.returncode != 0:
             raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
         os.replace(tmp, lib)
+    build_fastcall()
     return LIB
+
+
+FASTCALL_SRC = os.path.join(CSRC, "fastcall", "pa_fastcall.c")
+FASTCALL_LIB = os.path.join(HERE, "pa_fastcall.so")
+
+
+def build_fastcall():
+    """The CPython module the binding uses for its hottest calls instead of ctypes (csrc/fastcall): plain C
+    for the host, no GPU code.  The binding works without it, only slower, so a host without a C compiler
+    or Python's headers skips it with a note."""
+    import sysconfig
+    include = sysconfig.get_paths()["include"]
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None or not os.path.exists(os.path.join(include, "Python.h")):
+        print("build.py: no C compiler or no Python.h - pa_fastcall.so not built (the binding falls back to ctypes)",
+              file=sys.stderr)
+        return None
+    tmp = FASTCALL_LIB + ".tmp"
+    cmd = [cc, "-O2", "-Wall", "-shared", "-fPIC", "-I" + include, FASTCALL_SRC, "-o", tmp]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("compiling pa_fastcall failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-4000:]))
+    os.replace(tmp, FASTCALL_LIB)
+    return FASTCALL_LIB
 
 
 if __name__ == "__main__":

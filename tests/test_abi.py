@@ -54,3 +54,47 @@ def test_host_only_calls(lib):
     assert lib.pa_decode_noalloc(None, 0, 0, None, None, None, None, 0, None, 0, 0, None, None, 0, 4096, 16, 8,
                                  128, 16, 4, 1.0, 512, 64, 0, 0, 0, None) == -4
     assert b"scratch" in lib.pa_last_error()
+
+
+def test_fastcall_bindings_agree_with_ctypes(pa, lib):
+    """The hottest entry points are bound through pa_fastcall when it is built (always, after
+    __graft_entry__.build()): same addresses, same arguments, same return values and error texts as the
+    ctypes functions, and a TypeError / OverflowError where ctypes would have raised one."""
+    native = pa._native
+    assert os.path.exists(os.path.join(ROOT, "ai-infra-train-infer_amd", "pa_fastcall.so")), "run __graft_entry__.build()"
+    assert set(lib.fast_entries) == set(native.FAST_ENTRIES)
+    for name in native.FAST_ENTRIES:
+        assert getattr(lib, name) is not getattr(lib._cdll, name)
+    for name in set(native.SIGNATURES) - set(native.FAST_ENTRIES):
+        assert getattr(lib, name) is getattr(lib._cdll, name)
+    empty = (1234, 0, 2048, 1234, 1234, None, None, 0, 1234, 128, 128, 1234, 1234, 2048, 0, 16, 8, 128, 16, 100, 0.088,
+             0, 1, None, 0, 0, 0, 0, None)                                   # batch 0: returns before touching anything
+    cases = [("pa_decode", empty, 0)]
+    bad = list(empty)
+    bad[14] = -1
+    cases.append(("pa_decode", tuple(bad), -1))
+    cases.append(("pa_kv_store", (None, None, 0, 0, None, None, None, 4, 1024, 2, 64, None), -1))
+    cases.append(("pa_silu_mul", (None, 8, None, 8, None, 8, 0, 0, 8, None), 0))             # no rows
+    cases.append(("pa_silu_mul", (None, 8, None, 8, None, 8, 0, 3, 8, None), -1))            # null pointers
+    cases.append(("pa_add_rms_norm", (None, 8, None, 0, None, 0, 1e-6, None, 0, None, 8, 0, 3, 8, None), -1))
+    cases.append(("pa_sample", (None, 0, 0, 5, 7, 0.7, 0.9, None, None, None), -1))           # two floats in a row
+    for name, args, want in cases:
+        fast, slow = getattr(lib, name)(*args), getattr(lib._cdll, name)(*args)
+        assert fast == slow == want, (name, fast, slow)
+        if want:
+            getattr(lib, name)(*args)
+            text = lib.pa_last_error()
+            getattr(lib._cdll, name)(*args)
+            assert text == lib.pa_last_error() and name.encode() in text
+    with pytest.raises(TypeError):
+        lib.pa_decode(*empty[:-1])
+    with pytest.raises(TypeError):
+        lib.pa_decode(1.5, *empty[1:])
+    with pytest.raises(TypeError):
+        lib.pa_decode(*empty[:2], "2048", *empty[3:])
+    with pytest.raises(OverflowError):
+        lib.pa_decode(empty[0], 1 << 40, *empty[2:])
+    with pytest.raises(OverflowError):
+        lib.pa_decode(-5, *empty[1:])
+    # an int where a float goes is taken, as ctypes takes it
+    assert lib.pa_decode(*empty[:20], 1, *empty[21:]) == 0
