@@ -97,6 +97,8 @@ def _compile(hipcc, src):
 def build_library(force=True, verbose=False):
     """Compile and link the library. With force=False an up-to-date library is kept."""
     if not force and is_current():
+        if not os.path.exists(FASTCALL_LIB):
+            build_fastcall()
         return LIB
     hipcc = _hipcc()
     os.makedirs(OBJ, exist_ok=True)
