@@ -692,9 +692,9 @@ def choose_partition(batch, num_q_heads, num_kv_heads, max_context, head_dim=128
     over the CUs where whole rows of unequal length do not.  eager: the launch is issued call by call,
     not replayed from a graph, so a split also costs the host a second launch (it is then only taken
     where the single pass would last longer than the two calls take to issue)."""
-    bound, eighths = _known_lengths(max_context, longest_context, mean_context)
+    bound, fill = _known_lengths(max_context, longest_context, mean_context)
     return _choose_partition(batch, num_q_heads, num_kv_heads, bound, head_dim, kv_elem_bytes, compute_units,
-                             eighths, bool(eager))
+                             fill, bool(eager))
 
 
 def choose_launch(batch, num_q_heads, num_kv_heads, max_context, head_dim=128, kv_elem_bytes=2,
